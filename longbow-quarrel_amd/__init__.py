@@ -1,0 +1,17 @@
+"""longbow-quarrel on MI355X: a small model library with its own generation.
+
+One architecture (the Llama 3 dense decoder), one GPU, from a model folder
+(config.json + model.safetensors) to generated tokens, on hand-written gfx950
+kernels.
+"""
+from . import models  # noqa: F401  (registers the architectures)
+from .config import ConfigError, LlamaConfig, ModelConfig
+from .engine import Engine, StepEntry
+from .loading import load_engine, random_engine
+from .registry import register_architecture, registered_architectures
+from .weights import WeightError, write_model_folder
+
+__all__ = [
+    "ConfigError", "LlamaConfig", "ModelConfig", "Engine", "StepEntry", "load_engine", "random_engine",
+    "register_architecture", "registered_architectures", "WeightError", "write_model_folder",
+]

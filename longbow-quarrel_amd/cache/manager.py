@@ -1,0 +1,182 @@
+"""The cache: a slot for each live sequence, keys and values for each layer
+with each sequence's own length, and fixed-size state per sequence beside it.
+
+Layers are grouped by what their mixers need (`KVNeed`: kv heads, head size,
+window; `StateNeed`: a shape).  Every group has storage of its own: a pool of
+blocks of BLOCK_SIZE positions and a block table per slot, so a group that keeps
+all positions and a group that keeps a window of them never share rows.  The
+reference has one contiguous ring per layer for its single sequence
+(internal/engine/kv_cache_sliding_window.go:16-185) and a block-table variant
+it does not use (internal/engine/kv_cache_paged.go:17-278); a full cache here is
+an error, never an overwrite of old rows (internal/engine/kv_cache.go:121-124).
+
+Layouts of one layer of a group, chosen for the attention kernels:
+  K [blocks, kv_heads, BLOCK_SIZE, head_dim]   V [blocks, kv_heads, head_dim, BLOCK_SIZE]
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Mapping, Optional, Tuple
+
+import torch
+
+from ..parts.base import KVNeed, LayerCache, StateNeed
+from .slots import BLOCK_SIZE, CacheFull, FreeList
+
+
+def blocks_for(tokens: int) -> int:
+    return (tokens + BLOCK_SIZE - 1) // BLOCK_SIZE
+
+
+class KVGroup:
+    """Storage of the layers that share one KVNeed."""
+
+    def __init__(self, need: KVNeed, layers: List[int], n_blocks: int, max_slots: int,
+                 dtype: torch.dtype, device: torch.device) -> None:
+        self.need = need
+        self.layers = list(layers)
+        self.n_blocks = int(n_blocks)
+        self.max_slots = int(max_slots)
+        self.blocks = FreeList(self.n_blocks, "cache block")
+        shape_k = (len(layers), self.n_blocks, need.kv_heads, BLOCK_SIZE, need.head_dim)
+        shape_v = (len(layers), self.n_blocks, need.kv_heads, need.head_dim, BLOCK_SIZE)
+        # never read before written: reads are bounded by each sequence's length
+        self.k = torch.empty(shape_k, dtype=dtype, device=device)
+        self.v = torch.empty(shape_v, dtype=dtype, device=device)
+        self.table_width = max(1, self.n_blocks)
+        self.table_host = torch.zeros((self.max_slots, self.table_width), dtype=torch.int32)
+        self.table_dev = torch.zeros((self.max_slots, self.table_width), dtype=torch.int32, device=device)
+        # per slot: physical block of each logical block (None once trimmed away)
+        self.owned: List[List[Optional[int]]] = [[] for _ in range(self.max_slots)]
+
+    def layer_view(self, layer: int) -> LayerCache:
+        i = self.layers.index(layer)
+        return LayerCache(write=True, k=self.k[i], v=self.v[i], block_table=self.table_dev,
+                          block_size=BLOCK_SIZE)
+
+    def blocks_missing(self, slot: int, new_len: int) -> int:
+        return max(0, blocks_for(new_len) - len(self.owned[slot]))
+
+    def ensure(self, slot: int, new_len: int) -> None:
+        """Blocks for positions < new_len.  The caller has checked that enough are free."""
+        owned = self.owned[slot]
+        first = len(owned)
+        want = blocks_for(new_len)
+        if want <= first:
+            return
+        if want > self.table_width:
+            raise CacheFull(f"a sequence of {new_len} tokens needs {want} blocks, the table holds {self.table_width}")
+        owned.extend(self.blocks.take_many(want - first))
+        self.table_host[slot, first:want] = torch.tensor(owned[first:want], dtype=torch.int32)
+        self.table_dev[slot, first:want].copy_(self.table_host[slot, first:want])
+
+    def trim(self, slot: int, length: int) -> None:
+        """A windowed group gives back the blocks no later query can reach."""
+        w = self.need.window
+        if w <= 0:
+            return
+        first_needed = max(0, length - w + 1) // BLOCK_SIZE
+        owned = self.owned[slot]
+        for b in range(min(first_needed, len(owned))):
+            if owned[b] is not None:
+                self.blocks.give(owned[b])
+                owned[b] = None
+
+    def release(self, slot: int) -> None:
+        for b in self.owned[slot]:
+            if b is not None:
+                self.blocks.give(b)
+        self.owned[slot] = []
+
+
+class StateGroup:
+    """Fixed-size state of the layers that share one StateNeed: [layers, slots, *shape]."""
+
+    def __init__(self, need: StateNeed, layers: List[int], max_slots: int, device: torch.device) -> None:
+        self.need = need
+        self.layers = list(layers)
+        self.data = torch.zeros((len(layers), max_slots) + tuple(need.shape), dtype=need.dtype, device=device)
+
+    def layer_view(self, layer: int) -> LayerCache:
+        return LayerCache(write=True, state=self.data[self.layers.index(layer)])
+
+    def clear(self, slot: int) -> None:
+        self.data[:, slot].zero_()
+
+
+class CacheManager:
+    """Slots, key/value groups and state groups of one engine."""
+
+    def __init__(self, needs: Mapping[int, object], max_tokens: int, max_slots: int,
+                 dtype: torch.dtype, device: torch.device) -> None:
+        if max_tokens <= 0 or max_slots <= 0:
+            raise ValueError("the cache needs a positive number of tokens and slots")
+        self.max_tokens = int(max_tokens)
+        self.n_blocks = blocks_for(self.max_tokens)
+        self.max_slots = int(min(max_slots, self.n_blocks))
+        self.slots = FreeList(self.max_slots, "slot")
+        self.lengths = [0] * self.max_slots
+        self.kv_groups: List[KVGroup] = []
+        self.state_groups: List[StateGroup] = []
+        self._owner: Dict[int, object] = {}
+        by_need: Dict[object, List[int]] = {}
+        for layer in sorted(needs):
+            by_need.setdefault(needs[layer], []).append(layer)
+        for need, layers in by_need.items():
+            if isinstance(need, KVNeed):
+                g = KVGroup(need, layers, self.n_blocks, self.max_slots, dtype, device)
+                self.kv_groups.append(g)
+            elif isinstance(need, StateNeed):
+                g = StateGroup(need, layers, self.max_slots, device)
+                self.state_groups.append(g)
+            else:
+                raise TypeError(f"layer {layers[0]}: unknown cache need {need!r}")
+            for layer in layers:
+                self._owner[layer] = g
+
+    # ---- slots ------------------------------------------------------------------------
+    def acquire(self) -> int:
+        slot = self.slots.take()
+        self.lengths[slot] = 0
+        for g in self.state_groups:
+            g.clear(slot)
+        return slot
+
+    def release(self, slot: int) -> None:
+        self.slots.give(slot)  # raises if the slot is not in use
+        for g in self.kv_groups:
+            g.release(slot)
+        self.lengths[slot] = 0
+
+    def length(self, slot: int) -> int:
+        if not self.slots.is_taken(slot):
+            raise ValueError(f"slot {slot} is not in use")
+        return self.lengths[slot]
+
+    # ---- growth ---------------------------------------------------------------------------
+    def reserve(self, growth: Mapping[int, int]) -> None:
+        """Makes room for `growth[slot]` more tokens in every slot named, or raises CacheFull
+        before anything has changed."""
+        for g in self.kv_groups:
+            missing = sum(g.blocks_missing(slot, self.lengths[slot] + n) for slot, n in growth.items())
+            if missing > g.blocks.free_count:
+                raise CacheFull(
+                    f"the cache is full: {missing} more blocks of {BLOCK_SIZE} tokens are needed, "
+                    f"{g.blocks.free_count} of {g.n_blocks} are free")
+        for g in self.kv_groups:
+            for slot, n in growth.items():
+                g.ensure(slot, self.lengths[slot] + n)
+
+    def advance(self, growth: Mapping[int, int]) -> None:
+        for slot, n in growth.items():
+            self.lengths[slot] += n
+            for g in self.kv_groups:
+                g.trim(slot, self.lengths[slot])
+
+    # ---- views --------------------------------------------------------------------------------
+    def layer_views(self) -> Dict[int, LayerCache]:
+        return {layer: g.layer_view(layer) for layer, g in self._owner.items()}
+
+    def tokens_held(self) -> int:
+        """Tokens of live sequences, each rounded up to whole blocks (largest over the groups)."""
+        return max((g.blocks.taken_count for g in self.kv_groups), default=0) * BLOCK_SIZE

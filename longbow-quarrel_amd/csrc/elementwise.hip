@@ -1,0 +1,302 @@
+// Row-wise kernels of the decoder: embedding rows, RMSNorm (with the residual
+// add folded in), rotation + cache write, SwiGLU, residual add, row gather, casts.
+// Norm statistics, rotation angles and the residual sum are 32-bit (or wider).
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// out[r, :] = float(table[token[r], :])   (row copy, internal/device/kernels.metal:465-467)
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                             float* __restrict__ out, int D) {
+  const int r = blockIdx.x;
+  const long long tok = tokens[r];
+  const T* src = table + tok * (long long)D;
+  float* dst = out + (long long)r * D;
+  for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = to_f32(src[j]);
+}
+
+extern "C" int lq_embed(const void* table, int table_dtype, const int* tokens, float* out, int rows,
+                        int D, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && D > 0, "embed: rows %d and width %d must be positive", rows, D);
+  const int threads = D >= 1024 ? 256 : 64;
+  if (table_dtype == LQ_F32)
+    embed_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, tokens, out, D);
+  else if (table_dtype == LQ_BF16)
+    embed_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, tokens, out, D);
+  else
+    LQ_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
+  LQ_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------- RMSNorm
+// Per row: (x += delta, written back, if delta is given), s = sum x^2,
+// r = 1 / sqrt(s / D + eps), out = x * r * w.  eps inside the root, weight
+// after normalisation (internal/device/kernels.metal:905-942).
+template <typename TD, typename TO, bool HAS_DELTA>
+__global__ void rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                               const float* __restrict__ w, TO* __restrict__ out, int D, float eps) {
+  __shared__ float red[16];
+  const long long base = (long long)blockIdx.x * D;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < D; j += blockDim.x) {
+    float v = x[base + j];
+    if (HAS_DELTA) {
+      v += to_f32(delta[base + j]);
+      x[base + j] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)D + eps);
+  for (int j = threadIdx.x; j < D; j += blockDim.x) {
+    // each thread re-reads what it wrote itself: no barrier needed
+    out[base + j] = from_f32<TO>(x[base + j] * r * w[j]);
+  }
+}
+
+extern "C" int lq_rmsnorm(float* x, const void* delta, int delta_dtype, const float* w, float eps,
+                          void* out, int out_dtype, int rows, int D, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && D > 0, "rmsnorm: rows %d and width %d must be positive", rows, D);
+  LQ_REQUIRE(out_dtype == LQ_F32 || out_dtype == LQ_BF16, "rmsnorm: unknown out dtype %d", out_dtype);
+  const int threads = D >= 2048 ? 512 : (D >= 512 ? 256 : 64);
+#define LQ_NORM_LAUNCH(TD, TO, HAS)                                                         \
+  rmsnorm_kernel<TD, TO, HAS><<<rows, threads, 0, stream>>>(x, (const TD*)delta, w, (TO*)out, D, eps)
+  if (delta == nullptr) {
+    if (out_dtype == LQ_F32)
+      LQ_NORM_LAUNCH(float, float, false);
+    else
+      LQ_NORM_LAUNCH(float, bf16_t, false);
+  } else if (delta_dtype == LQ_F32) {
+    if (out_dtype == LQ_F32)
+      LQ_NORM_LAUNCH(float, float, true);
+    else
+      LQ_NORM_LAUNCH(float, bf16_t, true);
+  } else if (delta_dtype == LQ_BF16) {
+    if (out_dtype == LQ_F32)
+      LQ_NORM_LAUNCH(bf16_t, float, true);
+    else
+      LQ_NORM_LAUNCH(bf16_t, bf16_t, true);
+  } else {
+    LQ_REQUIRE(false, "rmsnorm: unknown delta dtype %d", delta_dtype);
+  }
+#undef LQ_NORM_LAUNCH
+  LQ_CHECK_LAUNCH("rmsnorm");
+  return 0;
+}
+
+// ---------------------------------------------------------------- residual add
+template <typename TD>
+__global__ void add_kernel(float* __restrict__ x, const TD* __restrict__ delta, long long n) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) x[i] += to_f32(delta[i]);
+}
+
+extern "C" int lq_add(float* x, const void* delta, int delta_dtype, long long n, hipStream_t stream) {
+  LQ_REQUIRE(n > 0, "add: count %lld must be positive", n);
+  const int threads = 256;
+  const int blocks = (int)(lq_ceil_div64(n, threads) < 8192 ? lq_ceil_div64(n, threads) : 8192);
+  if (delta_dtype == LQ_F32)
+    add_kernel<float><<<blocks, threads, 0, stream>>>(x, (const float*)delta, n);
+  else if (delta_dtype == LQ_BF16)
+    add_kernel<bf16_t><<<blocks, threads, 0, stream>>>(x, (const bf16_t*)delta, n);
+  else
+    LQ_REQUIRE(false, "add: unknown delta dtype %d", delta_dtype);
+  LQ_CHECK_LAUNCH("add");
+  return 0;
+}
+
+// ---------------------------------------------------------------- casts
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, long long n) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) out[i] = from_f32<TO>(to_f32(in[i]));
+}
+
+extern "C" int lq_cast(const void* in, int in_dtype, void* out, int out_dtype, long long n,
+                       hipStream_t stream) {
+  LQ_REQUIRE(n > 0, "cast: count %lld must be positive", n);
+  const int threads = 256;
+  const int blocks = (int)(lq_ceil_div64(n, threads) < 8192 ? lq_ceil_div64(n, threads) : 8192);
+  if (in_dtype == LQ_F32 && out_dtype == LQ_BF16)
+    cast_kernel<float, bf16_t><<<blocks, threads, 0, stream>>>((const float*)in, (bf16_t*)out, n);
+  else if (in_dtype == LQ_BF16 && out_dtype == LQ_F32)
+    cast_kernel<bf16_t, float><<<blocks, threads, 0, stream>>>((const bf16_t*)in, (float*)out, n);
+  else
+    LQ_REQUIRE(false, "cast: unsupported pair %d -> %d", in_dtype, out_dtype);
+  LQ_CHECK_LAUNCH("cast");
+  return 0;
+}
+
+// ---------------------------------------------------------------- SwiGLU
+// out[r, i] = silu(g) * u with g = gu[r, i], u = gu[r, I + i], silu(g) = g / (1 + e^-g).
+// No clamps (internal/device/cpu_ref.go:132-149).
+template <typename TI, typename TO>
+__global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int I, long long n) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    const long long r = i / I;
+    const int c = (int)(i - r * I);
+    const float g = to_f32(gu[r * 2 * I + c]);
+    const float u = to_f32(gu[r * 2 * I + I + c]);
+    out[i] = from_f32<TO>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int lq_swiglu(const void* gu, int in_dtype, void* out, int out_dtype, int rows, int I,
+                         hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && I > 0, "swiglu: rows %d and width %d must be positive", rows, I);
+  const long long n = (long long)rows * I;
+  const int threads = 256;
+  const int blocks = (int)(lq_ceil_div64(n, threads) < 16384 ? lq_ceil_div64(n, threads) : 16384);
+#define LQ_SWIGLU_LAUNCH(TI, TO) \
+  swiglu_kernel<TI, TO><<<blocks, threads, 0, stream>>>((const TI*)gu, (TO*)out, I, n)
+  if (in_dtype == LQ_F32 && out_dtype == LQ_F32)
+    LQ_SWIGLU_LAUNCH(float, float);
+  else if (in_dtype == LQ_F32 && out_dtype == LQ_BF16)
+    LQ_SWIGLU_LAUNCH(float, bf16_t);
+  else if (in_dtype == LQ_BF16 && out_dtype == LQ_BF16)
+    LQ_SWIGLU_LAUNCH(bf16_t, bf16_t);
+  else
+    LQ_REQUIRE(false, "swiglu: unsupported dtypes %d -> %d", in_dtype, out_dtype);
+#undef LQ_SWIGLU_LAUNCH
+  LQ_CHECK_LAUNCH("swiglu");
+  return 0;
+}
+
+// ---------------------------------------------------------------- row gather
+// out[i, :] = x[rows[i], :] (+ delta[rows[i], :]); picks the rows whose logits
+// are wanted before the final norm, carrying a not yet applied residual delta.
+template <typename TD, bool HAS_DELTA>
+__global__ void gather_rows_kernel(const float* __restrict__ x, const TD* __restrict__ delta,
+                                   const int* __restrict__ rows, float* __restrict__ out, int D) {
+  const long long src = (long long)rows[blockIdx.x] * D;
+  const long long dst = (long long)blockIdx.x * D;
+  for (int j = threadIdx.x; j < D; j += blockDim.x) {
+    float v = x[src + j];
+    if (HAS_DELTA) v += to_f32(delta[src + j]);
+    out[dst + j] = v;
+  }
+}
+
+extern "C" int lq_gather_rows(const float* x, const void* delta, int delta_dtype, const int* rows,
+                              float* out, int n, int D, hipStream_t stream) {
+  LQ_REQUIRE(n > 0 && D > 0, "gather_rows: count %d and width %d must be positive", n, D);
+  const int threads = D >= 1024 ? 256 : 64;
+  if (delta == nullptr)
+    gather_rows_kernel<float, false><<<n, threads, 0, stream>>>(x, nullptr, rows, out, D);
+  else if (delta_dtype == LQ_F32)
+    gather_rows_kernel<float, true><<<n, threads, 0, stream>>>(x, (const float*)delta, rows, out, D);
+  else if (delta_dtype == LQ_BF16)
+    gather_rows_kernel<bf16_t, true><<<n, threads, 0, stream>>>(x, (const bf16_t*)delta, rows, out, D);
+  else
+    LQ_REQUIRE(false, "gather_rows: unknown delta dtype %d", delta_dtype);
+  LQ_CHECK_LAUNCH("gather_rows");
+  return 0;
+}
+
+// ---------------------------------------------------------------- rotation + cache write
+// One block per row.  The row's position p comes from row_pos; its angles
+// p * f_i are formed in double from the double table f (hd/2 entries), so the
+// rotation is exact to 32-bit rounding at any position.  Pair (i, i + hd/2):
+//   x_i' = x_i cos - x_{i+hd/2} sin ; x_{i+hd/2}' = x_i sin + x_{i+hd/2} cos
+// (internal/device/kernels.metal:430-463).  q is rotated in place; rotated k
+// and plain v go to the paged cache (internal/device/kernels.metal:1736-1749
+// writes row p; here the row is found through the slot's block table):
+//   K[block][kv head][offset][hd]      V[block][kv head][hd][offset]
+// with block = table[slot][p / BS], offset = p % BS.
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                                  int ldq, int ldk, int ldv, int nh, int nkv, int hd,
+                                  const double* __restrict__ freqs, int has_rope,
+                                  const int* __restrict__ row_pos, const int* __restrict__ row_seq,
+                                  const int* __restrict__ seq_slot,
+                                  const int* __restrict__ block_table, int bt_stride,
+                                  T* __restrict__ kcache, T* __restrict__ vcache, int BS,
+                                  int store) {
+  extern __shared__ float cs[];  // cos[hd/2], sin[hd/2]
+  const int r = blockIdx.x;
+  const int half = hd / 2;
+  const int p = row_pos[r];
+  if (has_rope) {
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+      double s, c;
+      sincos((double)p * freqs[i], &s, &c);
+      cs[i] = (float)c;
+      cs[half + i] = (float)s;
+    }
+  } else {
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+      cs[i] = 1.0f;
+      cs[half + i] = 0.0f;
+    }
+  }
+  __syncthreads();
+
+  T* qr = q + (long long)r * ldq;
+  for (int idx = threadIdx.x; idx < nh * half; idx += blockDim.x) {
+    const int h = idx / half, i = idx - h * half;
+    const float x0 = to_f32(qr[h * hd + i]);
+    const float x1 = to_f32(qr[h * hd + i + half]);
+    const float c = cs[i], s = cs[half + i];
+    qr[h * hd + i] = from_f32<T>(x0 * c - x1 * s);
+    qr[h * hd + i + half] = from_f32<T>(x0 * s + x1 * c);
+  }
+  if (!store) return;
+
+  const int slot = seq_slot[row_seq[r]];
+  const long long blk = block_table[(long long)slot * bt_stride + p / BS];
+  const int off = p % BS;
+  const T* kr = k + (long long)r * ldk;
+  const T* vr = v + (long long)r * ldv;
+  for (int idx = threadIdx.x; idx < nkv * half; idx += blockDim.x) {
+    const int h = idx / half, i = idx - h * half;
+    const float x0 = to_f32(kr[h * hd + i]);
+    const float x1 = to_f32(kr[h * hd + i + half]);
+    const float c = cs[i], s = cs[half + i];
+    T* dst = kcache + ((blk * nkv + h) * BS + off) * (long long)hd;
+    dst[i] = from_f32<T>(x0 * c - x1 * s);
+    dst[i + half] = from_f32<T>(x0 * s + x1 * c);
+  }
+  for (int idx = threadIdx.x; idx < nkv * hd; idx += blockDim.x) {
+    const int h = idx / hd, d = idx - h * hd;
+    vcache[((blk * nkv + h) * hd + d) * (long long)BS + off] = vr[h * hd + d];
+  }
+}
+
+extern "C" int lq_rope_store(void* q, const void* k, const void* v, int dtype, int rows, int ldq,
+                             int ldk, int ldv, int nh, int nkv, int hd, const double* freqs,
+                             const int* row_pos, const int* row_seq, const int* seq_slot,
+                             const int* block_table, int bt_stride, void* kcache, void* vcache,
+                             int block_size, int store, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0, "rope_store: rows %d must be positive", rows);
+  LQ_REQUIRE(hd > 0 && hd % 2 == 0, "rope_store: head size %d must be even", hd);
+  LQ_REQUIRE(nh > 0 && nkv >= 0, "rope_store: head counts %d / %d", nh, nkv);
+  LQ_REQUIRE(ldq >= nh * hd, "rope_store: q row stride %d is less than %d", ldq, nh * hd);
+  if (store) {
+    LQ_REQUIRE(ldk >= nkv * hd && ldv >= nkv * hd, "rope_store: k/v row stride too small");
+    LQ_REQUIRE(block_size > 0 && bt_stride > 0, "rope_store: block size %d, table stride %d",
+               block_size, bt_stride);
+    LQ_REQUIRE(kcache && vcache && block_table && seq_slot && row_seq, "rope_store: null cache argument");
+  }
+  const int threads = 256;
+  const size_t smem = (size_t)hd * sizeof(float);
+  const int has_rope = freqs != nullptr;
+  if (dtype == LQ_F32)
+    rope_store_kernel<float><<<rows, threads, smem, stream>>>(
+        (float*)q, (const float*)k, (const float*)v, ldq, ldk, ldv, nh, nkv, hd, freqs, has_rope,
+        row_pos, row_seq, seq_slot, block_table, bt_stride, (float*)kcache, (float*)vcache,
+        block_size, store);
+  else if (dtype == LQ_BF16)
+    rope_store_kernel<bf16_t><<<rows, threads, smem, stream>>>(
+        (bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, ldq, ldk, ldv, nh, nkv, hd, freqs, has_rope,
+        row_pos, row_seq, seq_slot, block_table, bt_stride, (bf16_t*)kcache, (bf16_t*)vcache,
+        block_size, store);
+  else
+    LQ_REQUIRE(false, "rope_store: unknown dtype %d", dtype);
+  LQ_CHECK_LAUNCH("rope_store");
+  return 0;
+}

@@ -1,0 +1,266 @@
+"""The hand-written gfx950 kernels, bound through ctypes.
+
+`HipKernels` is the only compute backend of the library.  Every method checks
+on the host what its kernel and grid assume (dtype, device, contiguity, sizes),
+then launches on the current HIP stream.  There is no fallback: if the shared
+library cannot be built or loaded, constructing `HipKernels` raises.
+
+Tensors are torch tensors used as typed device buffers; no torch operator runs
+here.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_double, c_float, c_int, c_longlong, c_void_p
+from typing import Optional
+
+import torch
+
+from .. import build as _build
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelLibraryError(RuntimeError):
+    """The kernel library is missing, or a kernel refused its arguments."""
+
+
+_LIB = None
+
+
+def load_library() -> ctypes.CDLL:
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    try:
+        path = _build.ensure_built()
+    except Exception as e:  # BuildError, OSError
+        raise KernelLibraryError(
+            f"the gfx950 kernel library could not be built: {e}\n"
+            "This library has no CPU or library fallback; it needs hipcc (ROCm) to compile its kernels."
+        ) from e
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:
+        raise KernelLibraryError(f"cannot load {path}: {e}") from e
+    lib.lq_last_error.restype = ctypes.c_char_p
+    lib.lq_abi_version.restype = c_int
+    _LIB = lib
+    return lib
+
+
+def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelLibraryError(f"unsupported tensor dtype {t.dtype}") from None
+
+
+class HipKernels:
+    name = "hip-gfx950"
+
+    def __init__(self) -> None:
+        self.lib = load_library()
+        if not torch.cuda.is_available():
+            raise KernelLibraryError("no HIP device is visible; this library runs on a gfx950 GPU only")
+        self._stream: Optional[int] = None
+        self.force_generic = False  # route linear and attention to the size-agnostic kernels
+
+    # ------------------------------------------------------------------ plumbing
+    def use_stream(self, stream: Optional["torch.cuda.Stream"]) -> None:
+        """Launch on `stream` from now on (None: ask torch for its current stream each call)."""
+        self._stream = None if stream is None else int(stream.cuda_stream)
+
+    @property
+    def stream(self) -> c_void_p:
+        if self._stream is not None:
+            return c_void_p(self._stream)
+        return c_void_p(int(torch.cuda.current_stream().cuda_stream))
+
+    def _check(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelLibraryError(self.lib.lq_last_error().decode("utf-8", "replace"))
+
+    @staticmethod
+    def _dev(*tensors: Optional[torch.Tensor]) -> None:
+        for t in tensors:
+            if t is None:
+                continue
+            if not t.is_cuda:
+                raise KernelLibraryError("kernel arguments must live on the GPU")
+            if t.dim() > 0 and t.stride(-1) != 1 and t.shape[-1] != 1:
+                raise KernelLibraryError("kernel arguments must be contiguous in their last dimension")
+
+    @staticmethod
+    def _rows2d(t: torch.Tensor, what: str) -> int:
+        """Row stride in elements of a 2-D view whose last dimension is dense."""
+        if t.dim() != 2:
+            raise KernelLibraryError(f"{what}: expected a 2-D tensor, found shape {tuple(t.shape)}")
+        return int(t.stride(0)) if t.shape[0] > 1 else max(int(t.stride(0)), int(t.shape[1]))
+
+    @staticmethod
+    def _i32(t: torch.Tensor, what: str, n: int) -> None:
+        if t.dtype != torch.int32 or not t.is_contiguous() or t.numel() < n:
+            raise KernelLibraryError(f"{what}: need a contiguous int32 tensor of at least {n} entries")
+
+    # ------------------------------------------------------------------ kernels
+    def embed(self, table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+        """out[r, :] = float32(table[tokens[r], :])"""
+        self._dev(table, tokens, out)
+        rows, width = out.shape
+        self._i32(tokens, "embed tokens", rows)
+        if out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous():
+            raise KernelLibraryError("embed: out must be dense float32, the table dense")
+        if table.dim() != 2 or table.shape[1] != width:
+            raise KernelLibraryError(f"embed: table {tuple(table.shape)} does not match width {width}")
+        self._check(self.lib.lq_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(out),
+                                      c_int(rows), c_int(width), self.stream))
+
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+                delta: Optional[torch.Tensor] = None) -> None:
+        """(x += delta;) out = x / sqrt(mean(x^2) + eps) * weight, row by row; x is float32."""
+        self._dev(x, weight, out, delta)
+        rows, width = x.shape
+        if x.dtype != torch.float32 or not x.is_contiguous():
+            raise KernelLibraryError("rmsnorm: x must be dense float32")
+        if weight.dtype != torch.float32 or weight.numel() != width or not weight.is_contiguous():
+            raise KernelLibraryError(f"rmsnorm: weight must be float32 of {width} entries")
+        if tuple(out.shape) != (rows, width) or not out.is_contiguous():
+            raise KernelLibraryError("rmsnorm: out must be dense and shaped like x")
+        if delta is not None and (tuple(delta.shape) != (rows, width) or not delta.is_contiguous()):
+            raise KernelLibraryError("rmsnorm: delta must be dense and shaped like x")
+        self._check(self.lib.lq_rmsnorm(_ptr(x), _ptr(delta), c_int(_code(delta) if delta is not None else 0),
+                                        _ptr(weight), c_float(eps), _ptr(out), c_int(_code(out)),
+                                        c_int(rows), c_int(width), self.stream))
+
+    def add(self, x: torch.Tensor, delta: torch.Tensor) -> None:
+        """x += delta (x float32)."""
+        self._dev(x, delta)
+        if x.dtype != torch.float32 or x.shape != delta.shape or not x.is_contiguous() or not delta.is_contiguous():
+            raise KernelLibraryError("add: x must be dense float32 and delta dense of the same shape")
+        self._check(self.lib.lq_add(_ptr(x), _ptr(delta), c_int(_code(delta)), c_longlong(x.numel()), self.stream))
+
+    def cast(self, src: torch.Tensor, out: torch.Tensor) -> None:
+        self._dev(src, out)
+        if src.shape != out.shape or not src.is_contiguous() or not out.is_contiguous():
+            raise KernelLibraryError("cast: dense tensors of one shape are needed")
+        self._check(self.lib.lq_cast(_ptr(src), c_int(_code(src)), _ptr(out), c_int(_code(out)),
+                                     c_longlong(src.numel()), self.stream))
+
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+        """out[M, N] = x[M, K] . w[N, K]^T with 32-bit accumulation."""
+        self._dev(x, w, out)
+        if x.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+            raise KernelLibraryError("linear: 2-D tensors are needed")
+        m, k = x.shape
+        n = w.shape[0]
+        if w.shape[1] != k or tuple(out.shape) != (m, n):
+            raise KernelLibraryError(
+                f"linear: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+        if x.dtype != w.dtype:
+            raise KernelLibraryError(f"linear: x is {x.dtype} but w is {w.dtype}")
+        self._check(self.lib.lq_linear(_ptr(x), _ptr(w), _ptr(out), c_int(_code(x)), c_int(_code(out)),
+                                       c_int(m), c_int(n), c_int(k), c_int(self._rows2d(x, "x")),
+                                       c_int(self._rows2d(w, "w")), c_int(self._rows2d(out, "out")),
+                                       c_int(1 if self.force_generic else 0), self.stream))
+
+    def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
+        """out[r, i] = silu(gate_up[r, i]) * gate_up[r, I + i]"""
+        self._dev(gate_up, out)
+        rows, width = out.shape
+        if tuple(gate_up.shape) != (rows, 2 * width) or not gate_up.is_contiguous() or not out.is_contiguous():
+            raise KernelLibraryError("swiglu: gate_up must be dense [rows, 2 I] and out dense [rows, I]")
+        self._check(self.lib.lq_swiglu(_ptr(gate_up), c_int(_code(gate_up)), _ptr(out), c_int(_code(out)),
+                                       c_int(rows), c_int(width), self.stream))
+
+    def gather_rows(self, x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor,
+                    delta: Optional[torch.Tensor] = None) -> None:
+        """out[i, :] = x[rows[i], :] (+ delta[rows[i], :])"""
+        self._dev(x, rows, out, delta)
+        n, width = out.shape
+        self._i32(rows, "gather rows", n)
+        if x.dtype != torch.float32 or out.dtype != torch.float32 or x.shape[1] != width:
+            raise KernelLibraryError("gather_rows: float32 tensors of one width are needed")
+        if not x.is_contiguous() or not out.is_contiguous():
+            raise KernelLibraryError("gather_rows: dense tensors are needed")
+        if delta is not None and (delta.shape != x.shape or not delta.is_contiguous()):
+            raise KernelLibraryError("gather_rows: delta must be dense and shaped like x")
+        self._check(self.lib.lq_gather_rows(_ptr(x), _ptr(delta), c_int(_code(delta) if delta is not None else 0),
+                                            _ptr(rows), _ptr(out), c_int(n), c_int(width), self.stream))
+
+    def rope_store(self, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
+                   heads: int, kv_heads: int, head_dim: int, freqs: Optional[torch.Tensor],
+                   row_pos: torch.Tensor, row_seq: Optional[torch.Tensor] = None,
+                   seq_slot: Optional[torch.Tensor] = None, block_table: Optional[torch.Tensor] = None,
+                   kcache: Optional[torch.Tensor] = None, vcache: Optional[torch.Tensor] = None,
+                   block_size: int = 0) -> None:
+        """Rotate q (in place) and k by the rows' positions; write rotated k and v into the paged cache.
+
+        q [rows, >= heads*head_dim], k and v [rows, >= kv_heads*head_dim] (views into one buffer are
+        fine); freqs float64 [head_dim/2] or None for no rotation; without a cache only q is rotated.
+        """
+        self._dev(q, k, v, freqs, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
+        rows = q.shape[0]
+        store = kcache is not None
+        self._i32(row_pos, "row_pos", rows)
+        if q.shape[1] < heads * head_dim:
+            raise KernelLibraryError("rope_store: q is narrower than heads * head_dim")
+        if freqs is not None and (freqs.dtype != torch.float64 or freqs.numel() != head_dim // 2
+                                  or not freqs.is_contiguous()):
+            raise KernelLibraryError(f"rope_store: freqs must be float64 of {head_dim // 2} entries")
+        bt_stride = 1
+        if store:
+            if k is None or v is None or vcache is None or row_seq is None or seq_slot is None or block_table is None:
+                raise KernelLibraryError("rope_store: storing needs k, v, both caches and the batch's tables")
+            if k.dtype != q.dtype or v.dtype != q.dtype or kcache.dtype != q.dtype or vcache.dtype != q.dtype:
+                raise KernelLibraryError("rope_store: q, k, v and the caches must share one dtype")
+            if k.shape[0] != rows or v.shape[0] != rows or k.shape[1] < kv_heads * head_dim or v.shape[1] < kv_heads * head_dim:
+                raise KernelLibraryError("rope_store: k / v do not match the rows or kv width")
+            self._i32(row_seq, "row_seq", rows)
+            if seq_slot.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.dim() != 2:
+                raise KernelLibraryError("rope_store: seq_slot and block_table must be int32 (table 2-D)")
+            nb = kcache.shape[0]
+            if tuple(kcache.shape) != (nb, kv_heads, block_size, head_dim) or \
+                    tuple(vcache.shape) != (nb, kv_heads, head_dim, block_size) or \
+                    not kcache.is_contiguous() or not vcache.is_contiguous():
+                raise KernelLibraryError("rope_store: cache tensors do not have the paged layout")
+            bt_stride = int(block_table.stride(0))
+        self._check(self.lib.lq_rope_store(
+            _ptr(q), _ptr(k), _ptr(v), c_int(_code(q)), c_int(rows),
+            c_int(self._rows2d(q, "q")), c_int(self._rows2d(k, "k") if k is not None else 0),
+            c_int(self._rows2d(v, "v") if v is not None else 0),
+            c_int(heads), c_int(kv_heads if store else 0), c_int(head_dim), _ptr(freqs),
+            _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(block_table), c_int(bt_stride),
+            _ptr(kcache), _ptr(vcache), c_int(block_size), c_int(1 if store else 0), self.stream))
+
+    def attention(self, q: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
+                  row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor,
+                  block_table: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                  block_size: int, scale: float, window: int = 0) -> None:
+        """Causal grouped-query attention of the step's rows over their slots' cached keys."""
+        self._dev(q, out, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
+        rows = q.shape[0]
+        self._i32(row_pos, "row_pos", rows)
+        self._i32(row_seq, "row_seq", rows)
+        if out.shape[0] != rows or out.shape[1] < heads * head_dim or q.shape[1] < heads * head_dim:
+            raise KernelLibraryError("attention: q / out do not match rows x heads*head_dim")
+        if q.dtype != out.dtype or kcache.dtype != q.dtype or vcache.dtype != q.dtype:
+            raise KernelLibraryError("attention: q, out and the caches must share one dtype")
+        nb = kcache.shape[0]
+        if tuple(kcache.shape) != (nb, kv_heads, block_size, head_dim) or \
+                tuple(vcache.shape) != (nb, kv_heads, head_dim, block_size) or \
+                not kcache.is_contiguous() or not vcache.is_contiguous():
+            raise KernelLibraryError("attention: cache tensors do not have the paged layout")
+        if seq_slot.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.dim() != 2:
+            raise KernelLibraryError("attention: seq_slot and block_table must be int32 (table 2-D)")
+        self._check(self.lib.lq_attention(
+            _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")),
+            c_int(_code(q)), c_int(rows), c_int(heads), c_int(kv_heads), c_int(head_dim),
+            _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(block_table),
+            c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
+            c_float(scale), c_int(window), c_int(1 if self.force_generic else 0), self.stream))

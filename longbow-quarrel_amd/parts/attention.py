@@ -1,0 +1,87 @@
+"""Causal grouped-query attention over the paged cache.
+
+q = n Wq^T, k = n Wk^T, v = n Wv^T (no biases), heads are contiguous blocks of
+head_dim columns; q and k are position-encoded, k and v are written to the
+cache, each row attends to the keys of its own sequence up to its own position,
+then the output projection (internal/device/metal.go:1377-1430).  Query head h
+reads kv head h // (heads / kv_heads); scores are scaled by `scale`
+(1/sqrt(head_dim) in the reference, internal/device/kernels.metal:671-673).
+
+The three projection matrices are concatenated at bind time so that one matrix
+product makes q, k and v.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Mapping, Optional
+
+import torch
+
+from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mixer, PartSpec,
+                   StepContext, TensorSpec, build_part, project)
+
+
+@MIXERS.register("gqa_attention")
+class GQAttention(Mixer):
+    def __init__(self, width: int, heads: int, kv_heads: int, head_dim: int, position: PartSpec,
+                 prefix: str, scale: Optional[float] = None, window: int = 0,
+                 names: Optional[Mapping[str, str]] = None) -> None:
+        if heads % kv_heads != 0:
+            raise ValueError(f"{heads} heads cannot share {kv_heads} kv heads evenly")
+        self.width, self.heads, self.kv_heads, self.head_dim = int(width), int(heads), int(kv_heads), int(head_dim)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.window = int(window)
+        n = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
+        n.update(names or {})
+        self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
+        self.position = build_part(POSITION_ENCODINGS, position)
+        self.q_width = self.heads * self.head_dim
+        self.kv_width = self.kv_heads * self.head_dim
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [
+            TensorSpec(self.names["q"], (self.q_width, self.width)),
+            TensorSpec(self.names["k"], (self.kv_width, self.width)),
+            TensorSpec(self.names["v"], (self.kv_width, self.width)),
+            TensorSpec(self.names["o"], (self.width, self.q_width)),
+        ] + self.position.tensor_specs()
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        q, k, v = (tensors[self.names[key]] for key in ("q", "k", "v"))
+        if not (q.dtype == k.dtype == v.dtype):
+            raise ValueError(f"{self.names['q']}: q, k and v projections are stored in different dtypes")
+        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
+        self.w_o = tensors[self.names["o"]].contiguous()
+        self.position.bind(tensors, env)
+
+    def cache_need(self) -> KVNeed:
+        return KVNeed(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, cache: Optional[LayerCache]) -> torch.Tensor:
+        if cache is None or cache.k is None:
+            raise RuntimeError("attention needs a key/value cache")
+        kn = ctx.kernels
+        rows = h.shape[0]
+        qkv = ctx.ws.alloc((rows, self.q_width + 2 * self.kv_width), ctx.dtype)
+        project(kn, ctx, h, self.w_qkv, qkv)
+        q = qkv[:, : self.q_width]
+        k = qkv[:, self.q_width : self.q_width + self.kv_width]
+        v = qkv[:, self.q_width + self.kv_width :]
+        freqs = self.position.rotary_frequencies
+        if freqs is None:
+            self.position.apply(q, k, ctx)
+        if cache.write:
+            kn.rope_store(q, k, v, self.heads, self.kv_heads, self.head_dim, freqs, ctx.row_pos,
+                          ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size)
+        elif freqs is not None:
+            kn.rope_store(q, None, None, self.heads, 0, self.head_dim, freqs, ctx.row_pos)
+        att = ctx.ws.alloc((rows, self.q_width), ctx.dtype)
+        kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
+                     ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size,
+                     self.scale, self.window)
+        out = ctx.ws.alloc((rows, self.width), torch.float32)
+        project(kn, ctx, att, self.w_o, out)
+        return out

@@ -1,0 +1,292 @@
+"""Interfaces of the parts a model is put together from, and their registries.
+
+A model is data: a `ModelSpec` lists, layer by layer, which block, mixer,
+feed-forward, norm and position encoding to build and with which sizes and
+constants (`PartSpec(kind, params)`), plus the order in which layers run.  Each
+kind name maps to a class through a registry; registering another class under a
+new name is all it takes to make a new part available to any architecture.
+
+No part knows which model it is in: everything it needs comes through its
+constructor parameters, the tensors it declared, and the `StepContext`.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, Generic, List, Mapping, Optional, Tuple, TypeVar
+
+import torch
+
+T = TypeVar("T")
+
+
+class Registry(Generic[T]):
+    """Name -> class (or factory).  Unknown names fail with the list of known ones."""
+
+    def __init__(self, what: str) -> None:
+        self.what = what
+        self._items: Dict[str, T] = {}
+
+    def register(self, name: str, item: Optional[T] = None):
+        def put(obj: T) -> T:
+            if name in self._items and self._items[name] is not obj:
+                raise ValueError(f"{self.what} {name!r} is already registered")
+            self._items[name] = obj
+            return obj
+
+        return put if item is None else put(item)
+
+    def unregister(self, name: str) -> None:
+        self._items.pop(name, None)
+
+    def get(self, name: str) -> T:
+        if name not in self._items:
+            known = ", ".join(sorted(self._items)) or "none"
+            raise KeyError(f"unknown {self.what} {name!r}; registered: {known}")
+        return self._items[name]
+
+    def names(self) -> List[str]:
+        return sorted(self._items)
+
+    def __contains__(self, name: str) -> bool:
+        return name in self._items
+
+
+MIXERS: Registry = Registry("mixer")
+FEED_FORWARDS: Registry = Registry("feed-forward")
+NORMS: Registry = Registry("norm")
+POSITION_ENCODINGS: Registry = Registry("position encoding")
+BLOCKS: Registry = Registry("block")
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """Which class to build (`kind`, looked up in the part's registry) and its parameters."""
+
+    kind: str
+    params: Mapping[str, Any] = field(default_factory=dict)
+
+
+# ---- tensors a part binds -------------------------------------------------------
+
+#: follows the file: bfloat16 stays bfloat16, a 32-bit tensor stays 32-bit
+#: (float16 becomes bfloat16); everything becomes float32 in the float32 mode
+MATRIX = "matrix"
+#: always held in float32 (norm weights)
+VECTOR32 = "vector32"
+#: integer table, held as int32
+TABLE = "table"
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    name: str  # the safetensors name
+    shape: Tuple[int, ...]
+    kind: str = MATRIX
+    init: str = "normal"  # random-weights rule: "normal" | "ones" | "zeros"
+    optional: bool = False  # may be absent from the file (a tied head)
+
+
+# ---- what a mixer asks of the cache ----------------------------------------------
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """Keys and values per position: `kv_heads` x `head_dim` each; window = 0 keeps all positions,
+    window = w keeps the last w (older blocks go back to the pool)."""
+
+    kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A block of fixed size per sequence, zeroed when a slot is taken."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+# ---- build-time and step-time context ---------------------------------------------
+
+
+@dataclass
+class BuildEnv:
+    """What parts get when their tensors are bound."""
+
+    dtype: torch.dtype  # activation / cache dtype: torch.bfloat16 or torch.float32
+    device: torch.device
+    kernels: Any  # HipKernels, or a test's stand-in with the same methods
+
+
+class Workspace:
+    """Bump allocator over one device buffer; reset at the start of every step.
+
+    Addresses repeat from step to step for equal shapes, which a captured HIP
+    graph relies on.  It grows (outside captures) when a step needs more.
+    """
+
+    ALIGN = 256
+
+    def __init__(self, device: torch.device, nbytes: int = 1 << 20) -> None:
+        self.device = device
+        self.buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self.off = 0
+        self.high = 0
+        self.frozen = False  # set while a graph that uses this buffer is alive
+        self._spill: List[torch.Tensor] = []
+
+    def reset(self) -> None:
+        if self.high > self.buf.numel() and not self.frozen:
+            self.buf = torch.empty(int(self.high * 1.25) + self.ALIGN, dtype=torch.uint8, device=self.device)
+        self.off = 0
+        self.high = 0
+        self._spill = []
+
+    def alloc(self, shape, dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        start = (self.off + self.ALIGN - 1) // self.ALIGN * self.ALIGN
+        end = start + nbytes
+        self.off = end
+        self.high = max(self.high, end)
+        if end > self.buf.numel():
+            if self.frozen:
+                raise RuntimeError("workspace of a captured graph is too small for this step")
+            t = torch.empty(tuple(shape), dtype=dtype, device=self.device)  # this step only; reset() grows
+            self._spill.append(t)
+            return t
+        return self.buf[start:end].view(dtype).view(tuple(shape))
+
+
+@dataclass
+class StepContext:
+    """One step's batch as the parts see it.  Device arrays are int32."""
+
+    kernels: Any
+    dtype: torch.dtype
+    device: torch.device
+    ws: Workspace
+    rows: int  # tokens in this step, all sequences together (packed, no padding)
+    batch: int  # sequences in this step
+    tokens: torch.Tensor  # [rows]
+    row_seq: torch.Tensor  # [rows] index of the row's sequence within the batch
+    row_pos: torch.Tensor  # [rows] absolute position of the row in its sequence
+    seq_slot: torch.Tensor  # [batch] slot of each sequence
+    seq_start: torch.Tensor  # [batch] length before this step
+    seq_len: torch.Tensor  # [batch] length after this step
+    cu_rows: torch.Tensor  # [batch + 1] prefix sums of the rows per sequence
+    # host copies of the same (lists of ints), for launch shapes and for parts written with torch
+    host_slots: List[int] = field(default_factory=list)
+    host_start: List[int] = field(default_factory=list)
+    host_new: List[int] = field(default_factory=list)
+    max_new: int = 0
+    max_len: int = 0
+    decode: bool = False  # every sequence brings exactly one token
+
+
+@dataclass
+class LayerCache:
+    """The cache as one layer sees it."""
+
+    write: bool = True  # False when the layer reads the cache another layer filled
+    # keys/values (KVNeed)
+    k: Optional[torch.Tensor] = None  # [blocks, kv_heads, block_size, head_dim]
+    v: Optional[torch.Tensor] = None  # [blocks, kv_heads, head_dim, block_size]
+    block_table: Optional[torch.Tensor] = None  # int32 [slots, blocks per slot]
+    block_size: int = 0
+    # fixed-size state (StateNeed)
+    state: Optional[torch.Tensor] = None  # [slots, *shape]
+
+
+# ---- the parts -----------------------------------------------------------------------
+
+
+class Part:
+    """Declares the tensors it binds; receives them in `bind`."""
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return []
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        """`tensors` holds every declared name that the file had, already on the device
+        and in the dtype its kind asks for."""
+        self.env = env
+
+
+class Norm(Part):
+    """forward(x, ctx, delta=None) -> normalised activations [rows, width] in ctx.dtype.
+
+    x is the float32 residual stream; when `delta` is given it is first added
+    to x in place (the residual add of the sub-layer before, folded in)."""
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Either exposes `rotary_frequencies` (float64 [rot/2], half-split pairs) that the
+    attention kernel fuses with the cache write, or overrides `apply` to change q and k itself."""
+
+    rotary_frequencies: Optional[torch.Tensor] = None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor, ctx: StepContext) -> None:
+        """Encode positions into q [rows, heads*hd] and k [rows, kv_heads*hd] in place."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """forward(h, ctx, cache) -> [rows, width], what the block adds to the residual stream.
+
+    h are the normalised activations of the step's rows (packed; row r belongs
+    to sequence ctx.row_seq[r] at position ctx.row_pos[r]).  A mixer must give
+    the same result however a sequence's tokens are cut into steps."""
+
+    def cache_need(self):
+        """KVNeed, StateNeed or None."""
+        return None
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, cache: Optional[LayerCache]) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """forward(h, ctx) -> [rows, width]; row-independent."""
+
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arranges norm(s), mixer and feed-forward around the residual stream.
+
+    forward(x, pending, ctx, cache) -> pending': x is the float32 residual
+    stream [rows, width], updated in place; `pending` is a delta that still has
+    to be added to x (it lets the add ride on the next norm kernel).  The true
+    stream is x + pending."""
+
+    mixer: Mixer
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
+                cache: Optional[LayerCache]) -> Optional[torch.Tensor]:
+        raise NotImplementedError
+
+
+def build_part(registry: Registry, spec: PartSpec, **extra):
+    cls = registry.get(spec.kind)
+    return cls(**dict(spec.params), **extra)
+
+
+def project(kn, ctx: StepContext, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out = x . w^T.  A weight stored in 32-bit is used in 32-bit: bfloat16
+    activations are widened for it rather than the weight narrowed."""
+    if w.dtype == x.dtype:
+        kn.linear(x, w, out)
+        return
+    if w.dtype != torch.float32:
+        raise RuntimeError(f"a {w.dtype} weight cannot meet {x.dtype} activations")
+    wide = ctx.ws.alloc(x.shape, torch.float32)
+    kn.cast(x, wide)
+    kn.linear(wide, w, out)

@@ -1,0 +1,48 @@
+"""Dense SwiGLU feed-forward: down(silu(gate(n)) * up(n)), no biases, no clamps
+(internal/device/metal.go:1464-1471; silu(g) = g / (1 + e^-g),
+internal/device/cpu_ref.go:132-149).  gate and up are concatenated at bind time
+so that one matrix product makes both."""
+from __future__ import annotations
+
+from typing import Dict, List, Mapping, Optional
+
+import torch
+
+from .base import FEED_FORWARDS, BuildEnv, FeedForward, StepContext, TensorSpec, project
+
+
+@FEED_FORWARDS.register("swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, width: int, inner: int, prefix: str, names: Optional[Mapping[str, str]] = None) -> None:
+        self.width, self.inner = int(width), int(inner)
+        n = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+        n.update(names or {})
+        self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [
+            TensorSpec(self.names["gate"], (self.inner, self.width)),
+            TensorSpec(self.names["up"], (self.inner, self.width)),
+            TensorSpec(self.names["down"], (self.width, self.inner)),
+        ]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        gate, up = tensors[self.names["gate"]], tensors[self.names["up"]]
+        if gate.dtype != up.dtype:
+            raise ValueError(f"{self.names['gate']}: gate and up projections are stored in different dtypes")
+        self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
+        self.w_down = tensors[self.names["down"]].contiguous()
+
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        kn = ctx.kernels
+        rows = h.shape[0]
+        gu = ctx.ws.alloc((rows, 2 * self.inner), torch.float32)
+        project(kn, ctx, h, self.w_gate_up, gu)
+        act = ctx.ws.alloc((rows, self.inner), ctx.dtype)
+        kn.swiglu(gu, act)
+        out = ctx.ws.alloc((rows, self.width), torch.float32)
+        project(kn, ctx, act, self.w_down, out)
+        return out
