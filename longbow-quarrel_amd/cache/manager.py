@@ -40,9 +40,10 @@ class KVGroup:
         self.blocks = FreeList(self.n_blocks, "cache block")
         shape_k = (len(layers), self.n_blocks, need.kv_heads, BLOCK_SIZE, need.head_dim)
         shape_v = (len(layers), self.n_blocks, need.kv_heads, need.head_dim, BLOCK_SIZE)
-        # never read before written: reads are bounded by each sequence's length
-        self.k = torch.empty(shape_k, dtype=dtype, device=device)
-        self.v = torch.empty(shape_v, dtype=dtype, device=device)
+        # reads are bounded by each sequence's length, but kernels load whole tiles of a block and
+        # mask afterwards: what they load must at least be finite numbers
+        self.k = torch.zeros(shape_k, dtype=dtype, device=device)
+        self.v = torch.zeros(shape_v, dtype=dtype, device=device)
         self.table_width = max(1, self.n_blocks)
         self.table_host = torch.zeros((self.max_slots, self.table_width), dtype=torch.int32)
         self.table_dev = torch.zeros((self.max_slots, self.table_width), dtype=torch.int32, device=device)

@@ -1,0 +1,276 @@
+// bfloat16 matrix products on the gfx950 matrix cores:  C[M, N] = A[M, K] . W[N, K]^T.
+//
+// Both operands have K contiguous, which is what the MFMA operand layout
+// wants: a lane holds 8 consecutive k of one row (A) or one column (W row).
+//
+//   v_mfma_f32_32x32x16_bf16: lane l gives A[row l%32][k (l/32)*8 .. +8] and
+//     B[col l%32][k (l/32)*8 .. +8]; it receives D[(e/4)*8 + (l/32)*4 + e%4][l%32], e < 16.
+//   v_mfma_f32_16x16x32_bf16: lane l gives A[row l%16][k (l/16)*8 .. +8] and
+//     B[col l%16][same k]; it receives D[(l/16)*4 + e][l%16], e < 4.
+//
+// Two kernels:
+//  * tiled: a block of 4 waves (2 x 2) computes a (2*WM*32) x (2*WN*32) tile, operands staged
+//    through padded LDS in steps of 64 k, next step prefetched into registers while the current one
+//    is multiplied.  For many rows (prefill).
+//  * skinny: at most 16 rows (decode).  A block owns 16 output columns; its KW waves split K,
+//    stream their slice of the 16 weight rows straight from memory into MFMA operands (every
+//    weight byte is read once, 16 bytes a lane), and add their partial tiles through LDS in
+//    wave order, so the result does not depend on timing.
+//
+// Accumulation is 32-bit.  K must be a multiple of 8 and rows 16-byte aligned; the dispatcher
+// sends everything else to the size-agnostic kernel.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+__device__ inline bf16x8 as_bf16x8(u32x4 v) {
+  union {
+    u32x4 u;
+    bf16x8 b;
+  } c;
+  c.u = v;
+  return c.b;
+}
+
+template <typename TO>
+__device__ inline void store_out(TO* p, float v);
+template <>
+__device__ inline void store_out<float>(float* p, float v) {
+  *p = v;
+}
+template <>
+__device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
+  *p = f32_to_bf16(v);
+}
+
+// ------------------------------------------------------------------ tiled
+constexpr int TBK = 64;           // k per stage
+constexpr int TLD = TBK + 8;      // padded LDS row, in elements (144 bytes: conflict-free b128 reads)
+
+template <int WM, int WN, typename TO>
+__global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A, int lda,
+                                                              const bf16_t* __restrict__ W, int ldw,
+                                                              TO* __restrict__ C, int ldc, int M, int N,
+                                                              int K, int tiles_m, int tiles_n) {
+  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  constexpr int A_CHUNKS = BM * (TBK / 8) / 256;  // 16-byte chunks a thread loads per stage
+  constexpr int W_CHUNKS = BN * (TBK / 8) / 256;
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  uint16_t* As = lds;                 // [BM][TLD]
+  uint16_t* Ws = lds + BM * TLD;      // [BN][TLD]
+
+  // Consecutive blocks go to different XCDs (8 of them, each with its own L2).  Remap so that
+  // one XCD gets a contiguous run of tiles, and let a run walk the m-tiles of one n-tile first:
+  // its blocks then share the same weight tile in that XCD's L2.
+  const int total = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  if (total % 8 == 0) pid = (pid % 8) * (total / 8) + pid / 8;  // ragged runs keep the plain order
+  const int tm = pid % tiles_m, tn = pid / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  u32x4 ra[A_CHUNKS], rw[W_CHUNKS];
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  auto load_stage = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const int c = tid + i * 256;
+      const int row = c >> 3, kc = (c & 7) * 8;
+      const int m = min(m0 + row, M - 1);
+      ra[i] = (k0 + kc < K) ? *(const u32x4*)(A + (long long)m * lda + k0 + kc) : zero;
+    }
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) {
+      const int c = tid + i * 256;
+      const int row = c >> 3, kc = (c & 7) * 8;
+      const int n = min(n0 + row, N - 1);
+      rw[i] = (k0 + kc < K) ? *(const u32x4*)(W + (long long)n * ldw + k0 + kc) : zero;
+    }
+  };
+  auto store_stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const int c = tid + i * 256;
+      *(u32x4*)(As + (c >> 3) * TLD + (c & 7) * 8) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) {
+      const int c = tid + i * 256;
+      *(u32x4*)(Ws + (c >> 3) * TLD + (c & 7) * 8) = rw[i];
+    }
+  };
+
+  load_stage(0);
+  for (int k0 = 0; k0 < K; k0 += TBK) {
+    __syncthreads();  // everyone is done reading the previous stage
+    store_stage();
+    __syncthreads();
+    if (k0 + TBK < K) load_stage(k0 + TBK);  // in flight while this stage is multiplied
+#pragma unroll
+    for (int kk = 0; kk < TBK / 16; ++kk) {
+      bf16x8 a[WM], b[WN];
+      const int koff = kk * 16 + (lane >> 5) * 8;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        a[i] = as_bf16x8(*(const u32x4*)(As + (wm * WM * 32 + i * 32 + (lane & 31)) * TLD + koff));
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        b[j] = as_bf16x8(*(const u32x4*)(Ws + (wn * WN * 32 + j * 32 + (lane & 31)) * TLD + koff));
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int col = n0 + wn * WN * 32 + j * 32 + (lane & 31);
+      if (col >= N) continue;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * WM * 32 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row < M) store_out<TO>(C + (long long)row * ldc + col, acc[i][j][e]);
+      }
+    }
+}
+
+template <int WM, int WN, typename TO>
+int launch_tiled(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
+                 hipStream_t stream) {
+  constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
+  const int tiles_m = lq_ceil_div(M, BM), tiles_n = lq_ceil_div(N, BN);
+  const size_t smem = (size_t)(BM + BN) * TLD * sizeof(uint16_t);
+  auto kernel = gemm_bf16_tiled_kernel<WM, WN, TO>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)smem);
+    if (e != hipSuccess) {
+      lq_set_error("linear: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+      return -2;
+    }
+    configured = true;
+  }
+  const long long blocks = (long long)tiles_m * tiles_n;
+  LQ_REQUIRE(blocks < (1ll << 31), "linear: too many tiles");
+  kernel<<<(int)blocks, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, (TO*)C, ldc,
+                                              M, N, K, tiles_m, tiles_n);
+  LQ_CHECK_LAUNCH("linear(mfma tiled)");
+  return 0;
+}
+
+// ------------------------------------------------------------------ skinny (M <= 16)
+constexpr int SK_UNROLL = 4;  // 64-k chunks a wave keeps in flight (8 weight loads of 1 KiB)
+
+template <int KW, typename TO>
+__global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
+                                                                   const bf16_t* __restrict__ W, int ldw,
+                                                                   TO* __restrict__ C, int ldc, int M,
+                                                                   int N, int K) {
+  __shared__ float red[KW][256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * 16;
+  const int g = lane >> 4;
+  const int nrow = min(n0 + (lane & 15), N - 1);
+  const int mrow = min(lane & 15, M - 1);
+  const bf16_t* wp = W + (long long)nrow * ldw + g * 8;
+  const bf16_t* xp = X + (long long)mrow * ldx + g * 8;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  // wave w takes 64-k chunks w, w + KW, w + 2 KW, ... : the block reads KW * 128 bytes of every
+  // weight row at a time
+  for (int kc = wave * 64; kc < K; kc += KW * 64 * SK_UNROLL) {
+    u32x4 wv[SK_UNROLL][2], xv[SK_UNROLL][2];
+#pragma unroll
+    for (int u = 0; u < SK_UNROLL; ++u) {
+      const int k = kc + u * KW * 64;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const bool ok = k + h * 32 + g * 8 < K;
+        wv[u][h] = ok ? __builtin_nontemporal_load((const u32x4*)(wp + k + h * 32)) : zero;
+        xv[u][h] = ok ? *(const u32x4*)(xp + k + h * 32) : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < SK_UNROLL; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[u][h]), as_bf16x8(wv[u][h]), acc, 0, 0, 0);
+  }
+  // acc[e] = C[(lane / 16) * 4 + e][n0 + lane % 16], partial over this wave's k
+#pragma unroll
+  for (int e = 0; e < 4; ++e) red[wave][e * 64 + lane] = acc[e];
+  __syncthreads();
+  if (wave == 0) {
+    const int col = n0 + (lane & 15);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < KW; ++w) s += red[w][e * 64 + lane];
+      const int row = g * 4 + e;
+      if (row < M && col < N) store_out<TO>(C + (long long)row * ldc + col, s);
+    }
+  }
+}
+
+template <int KW, typename TO>
+int launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc,
+                  hipStream_t stream) {
+  gemm_bf16_skinny_kernel<KW, TO><<<lq_ceil_div(N, 16), KW * 64, 0, stream>>>(
+      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K);
+  LQ_CHECK_LAUNCH("linear(mfma skinny)");
+  return 0;
+}
+
+template <typename TO>
+int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
+             hipStream_t stream) {
+  if (M <= 16) {
+    // enough waves to keep the memory system busy: about 8 a CU
+    const long long tiles = lq_ceil_div(N, 16);
+    const int chunks = lq_ceil_div(K, 64);
+    if (tiles * 4 >= 2048 || chunks < 8) return launch_skinny<4, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (tiles * 8 >= 2048 || chunks < 16) return launch_skinny<8, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    return launch_skinny<16, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  }
+  if (M <= 64) return launch_tiled<1, 2, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  return launch_tiled<2, 2, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+}
+
+}  // namespace
+
+// Whether the MFMA kernels take this problem (the caller falls back to the generic kernel if not).
+bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int lda, int ldw) {
+  return in_dtype == LQ_BF16 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 &&
+         ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
+}
+
+int lq_gemm_mfma(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K, int lda,
+                 int ldw, int ldc, hipStream_t stream) {
+  if (out_dtype == LQ_F32) return dispatch<float>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  if (out_dtype == LQ_BF16) return dispatch<bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  lq_set_error("linear: unknown out dtype %d", out_dtype);
+  return -1;
+}

@@ -238,15 +238,31 @@ class HipKernels:
             _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(block_table), c_int(bt_stride),
             _ptr(kcache), _ptr(vcache), c_int(block_size), c_int(1 if store else 0), self.stream))
 
+    def attention_workspace(self, dtype: torch.dtype, rows: int, heads: int, kv_heads: int, head_dim: int,
+                            block_size: int, decode: bool, max_len: int) -> int:
+        """Float32 entries of scratch that `attention` wants for this launch (0: none)."""
+        self.lib.lq_attention_workspace.restype = c_longlong
+        if self.force_generic or dtype not in _DTYPE_CODE:
+            return 0
+        return int(self.lib.lq_attention_workspace(c_int(_DTYPE_CODE[dtype]), c_int(rows), c_int(heads),
+                                                   c_int(kv_heads), c_int(head_dim), c_int(block_size),
+                                                   c_int(1 if decode else 0), c_int(max_len)))
+
     def attention(self, q: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
-                  row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor,
+                  row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor, cu_rows: torch.Tensor,
                   block_table: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
-                  block_size: int, scale: float, window: int = 0) -> None:
-        """Causal grouped-query attention of the step's rows over their slots' cached keys."""
-        self._dev(q, out, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
+                  block_size: int, scale: float, window: int = 0, decode: bool = False, max_len: int = 0,
+                  workspace: Optional[torch.Tensor] = None) -> None:
+        """Causal grouped-query attention of the step's rows over their slots' cached keys.
+
+        `decode` promises one row per sequence; `max_len` is then an upper bound of the lengths
+        after this step and `workspace` float32 scratch of `attention_workspace(...)` entries."""
+        self._dev(q, out, row_pos, row_seq, seq_slot, cu_rows, block_table, kcache, vcache, workspace)
         rows = q.shape[0]
+        batch = seq_slot.numel()
         self._i32(row_pos, "row_pos", rows)
         self._i32(row_seq, "row_seq", rows)
+        self._i32(cu_rows, "cu_rows", batch + 1)
         if out.shape[0] != rows or out.shape[1] < heads * head_dim or q.shape[1] < heads * head_dim:
             raise KernelLibraryError("attention: q / out do not match rows x heads*head_dim")
         if q.dtype != out.dtype or kcache.dtype != q.dtype or vcache.dtype != q.dtype:
@@ -258,9 +274,17 @@ class HipKernels:
             raise KernelLibraryError("attention: cache tensors do not have the paged layout")
         if seq_slot.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.dim() != 2:
             raise KernelLibraryError("attention: seq_slot and block_table must be int32 (table 2-D)")
+        if decode and rows != batch:
+            raise KernelLibraryError("attention: decode means one row per sequence")
+        ws_n = 0
+        if workspace is not None:
+            if workspace.dtype != torch.float32 or not workspace.is_contiguous():
+                raise KernelLibraryError("attention: workspace must be dense float32")
+            ws_n = workspace.numel()
         self._check(self.lib.lq_attention(
             _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")),
-            c_int(_code(q)), c_int(rows), c_int(heads), c_int(kv_heads), c_int(head_dim),
-            _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(block_table),
+            c_int(_code(q)), c_int(rows), c_int(batch), c_int(heads), c_int(kv_heads), c_int(head_dim),
+            _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(cu_rows), _ptr(block_table),
             c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
-            c_float(scale), c_int(window), c_int(1 if self.force_generic else 0), self.stream))
+            c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
+            c_longlong(ws_n), c_int(1 if self.force_generic else 0), self.stream))

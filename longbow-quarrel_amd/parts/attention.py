@@ -79,9 +79,12 @@ class GQAttention(Mixer):
         elif freqs is not None:
             kn.rope_store(q, None, None, self.heads, 0, self.head_dim, freqs, ctx.row_pos)
         att = ctx.ws.alloc((rows, self.q_width), ctx.dtype)
+        need = kn.attention_workspace(ctx.dtype, rows, self.heads, self.kv_heads, self.head_dim,
+                                      cache.block_size, ctx.decode, ctx.max_len)
+        scratch = ctx.ws.alloc((need,), torch.float32) if need else None
         kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
-                     ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size,
-                     self.scale, self.window)
+                     ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
+                     self.scale, self.window, decode=ctx.decode, max_len=ctx.max_len, workspace=scratch)
         out = ctx.ws.alloc((rows, self.width), torch.float32)
         project(kn, ctx, att, self.w_o, out)
         return out

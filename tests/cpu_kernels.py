@@ -84,8 +84,11 @@ class CpuKernels:
             kcache[blk, :, off, :] = kr[r]
             vcache[blk, :, :, off] = vr[r]
 
-    def attention(self, q, out, heads, kv_heads, head_dim, row_pos, row_seq, seq_slot, block_table,
-                  kcache, vcache, block_size, scale, window=0):
+    def attention_workspace(self, dtype, rows, heads, kv_heads, head_dim, block_size, decode, max_len):
+        return 0
+
+    def attention(self, q, out, heads, kv_heads, head_dim, row_pos, row_seq, seq_slot, cu_rows, block_table,
+                  kcache, vcache, block_size, scale, window=0, decode=False, max_len=0, workspace=None):
         rows = q.shape[0]
         group = heads // kv_heads
         for r in range(rows):

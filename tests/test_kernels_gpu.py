@@ -1,0 +1,306 @@
+"""Each HIP kernel alone against a plain float64 expression of the same formula,
+at sizes other than the tiny models' (odd widths, 8B-shaped rows, long key ranges)."""
+import math
+
+import pytest
+import torch
+
+import plain
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def kn():
+    from longbow_quarrel_amd.kernels.hip import HipKernels
+
+    return HipKernels()
+
+
+def rnd(shape, seed, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def i32(values):
+    return torch.tensor(list(values), dtype=torch.int32, device=DEV)
+
+
+# --------------------------------------------------------------------------- rows
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [331, 4096])
+def test_embed(kn, dtype, width):
+    table = rnd((97, width), 1, dtype)
+    toks = i32([5, 96, 0, 5, 33])
+    out = torch.empty((5, width), dtype=torch.float32, device=DEV)
+    kn.embed(table, toks, out)
+    assert torch.equal(out, table[toks.long()].float())
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width,eps", [(2, 4096, 1e-5), (7, 331, 3e-6), (1, 64, 1e-6), (3, 5000, 1e-5)])
+def test_rmsnorm(kn, out_dtype, rows, width, eps):
+    x = rnd((rows, width), 2, scale=5.0)
+    w = rnd((width,), 3).abs() * 2
+    out = torch.empty((rows, width), dtype=out_dtype, device=DEV)
+    kn.rmsnorm(x, w, eps, out)
+    want = plain.rms_norm(x.cpu(), w.cpu(), eps)
+    assert rel_err(out, want) < (2e-6 if out_dtype == torch.float32 else 5e-3)
+
+
+@pytest.mark.parametrize("delta_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_folds_the_residual_add(kn, delta_dtype):
+    x = rnd((5, 777), 4)
+    d = rnd((5, 777), 5, delta_dtype)
+    w = rnd((777,), 6)
+    x0 = x.clone()
+    out = torch.empty((5, 777), dtype=torch.float32, device=DEV)
+    kn.rmsnorm(x, w, 1e-5, out, delta=d)
+    summed = x0.double() + d.double()
+    assert rel_err(x, summed) < 1e-6  # the stream itself carries the sum on
+    assert rel_err(out, plain.rms_norm(summed.cpu(), w.cpu(), 1e-5)) < 2e-6
+
+
+def test_add_cast_gather(kn):
+    x = rnd((9, 130), 7)
+    d = rnd((9, 130), 8, torch.bfloat16)
+    x0 = x.clone()
+    kn.add(x, d)
+    assert torch.equal(x, x0 + d.float())
+    b = torch.empty_like(x, dtype=torch.bfloat16)
+    kn.cast(x, b)
+    assert torch.equal(b, x.to(torch.bfloat16))
+    f = torch.empty_like(x)
+    kn.cast(b, f)
+    assert torch.equal(f, b.float())
+    rows = i32([8, 0, 3])
+    out = torch.empty((3, 130), dtype=torch.float32, device=DEV)
+    kn.gather_rows(x, rows, out)
+    assert torch.equal(out, x[rows.long()])
+    kn.gather_rows(x, rows, out, delta=d)
+    assert torch.equal(out, (x + d.float())[rows.long()])
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(kn, out_dtype):
+    gu = rnd((6, 2 * 333), 9, scale=3.0)
+    out = torch.empty((6, 333), dtype=out_dtype, device=DEV)
+    kn.swiglu(gu, out)
+    want = plain.swiglu(gu[:, :333].cpu(), gu[:, 333:].cpu())
+    assert rel_err(out, want) < (2e-6 if out_dtype == torch.float32 else 5e-3)
+
+
+# --------------------------------------------------------------------------- linear
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (5, 331, 80), (70, 130, 333), (129, 65, 17), (3, 1000, 4096)])
+def test_linear_float32(kn, m, n, k):
+    x, w = rnd((m, k), 10), rnd((n, k), 11)
+    out = torch.empty((m, n), dtype=torch.float32, device=DEV)
+    kn.linear(x, w, out)
+    want = x.double().cpu() @ w.double().cpu().t()
+    assert rel_err(out, want) < 2e-6
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [
+    (1, 4096, 4096), (8, 6144, 4096), (16, 1000, 14336), (3, 40, 72), (13, 17, 8),       # skinny
+    (17, 256, 128), (64, 130, 264), (100, 300, 1000), (128, 128, 64), (257, 515, 4096),  # tiled
+    (2048, 1024, 512),
+])
+def test_linear_bfloat16_matrix_cores(kn, out_dtype, m, n, k):
+    x, w = rnd((m, k), 12, torch.bfloat16), rnd((n, k), 13, torch.bfloat16)
+    out = torch.empty((m, n), dtype=out_dtype, device=DEV)
+    kn.linear(x, w, out)
+    want = x.double().cpu() @ w.double().cpu().t()
+    # float32 accumulation of exact bfloat16 products: only the output rounding is bfloat16-sized
+    assert rel_err(out, want) < (1e-5 if out_dtype == torch.float32 else 5e-3)
+
+
+def test_linear_bfloat16_odd_k_takes_the_generic_kernel(kn):
+    x, w = rnd((9, 77), 14, torch.bfloat16), rnd((33, 77), 15, torch.bfloat16)
+    out = torch.empty((9, 33), dtype=torch.float32, device=DEV)
+    kn.linear(x, w, out)
+    assert rel_err(out, x.double().cpu() @ w.double().cpu().t()) < 1e-5
+
+
+def test_linear_row_does_not_depend_on_the_batch(kn):
+    """Row 0 alone (skinny kernel) against row 0 among 300 (tiled kernel): equal up to float32 rounding."""
+    x, w = rnd((300, 4096), 16, torch.bfloat16), rnd((512, 4096), 17, torch.bfloat16)
+    big = torch.empty((300, 512), dtype=torch.float32, device=DEV)
+    one = torch.empty((1, 512), dtype=torch.float32, device=DEV)
+    kn.linear(x, w, big)
+    kn.linear(x[:1], w, one)
+    assert rel_err(one, big[:1]) < 1e-5
+
+
+# --------------------------------------------------------------------------- rotation + cache write, attention
+
+BS = 64
+
+
+def paged_cache(lengths, kv_heads, head_dim, dtype, seed):
+    """Random keys/values for sequences of the given lengths in a paged cache whose blocks are
+    handed out in a shuffled order; returns dense copies too."""
+    g = torch.Generator().manual_seed(seed)
+    need = [(n + BS - 1) // BS for n in lengths]
+    n_blocks = sum(need) + 3
+    perm = torch.randperm(n_blocks, generator=g).tolist()
+    table = torch.zeros((len(lengths) + 2, max(need) + 1), dtype=torch.int32)
+    slots = list(range(len(lengths), 0, -1))  # slot ids differ from batch indices
+    kc = torch.zeros((n_blocks, kv_heads, BS, head_dim), dtype=dtype)
+    vc = torch.zeros((n_blocks, kv_heads, head_dim, BS), dtype=dtype)
+    dense = []
+    for b, n in enumerate(lengths):
+        k = torch.randn((n, kv_heads, head_dim), generator=g).to(dtype)
+        v = torch.randn((n, kv_heads, head_dim), generator=g).to(dtype)
+        dense.append((k, v))
+        for j in range(need[b]):
+            blk = perm.pop()
+            table[slots[b], j] = blk
+            lo, hi = j * BS, min(n, (j + 1) * BS)
+            kc[blk, :, : hi - lo, :] = k[lo:hi].transpose(0, 1)
+            vc[blk, :, :, : hi - lo] = v[lo:hi].permute(1, 2, 0)
+    return kc.to(DEV), vc.to(DEV), table.to(DEV), slots, dense
+
+
+def run_attention(kn, q_rows, lengths, new, heads, kv_heads, head_dim, dtype, seed, window=0, decode=False,
+                  force_generic=False, standout=None):
+    """q rows for the last `new[b]` positions of each sequence; returns (got, want)."""
+    kc, vc, table, slots, dense = paged_cache(lengths, kv_heads, head_dim, dtype, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    rows = sum(new)
+    q = torch.randn((rows, heads * head_dim), generator=g).to(dtype)
+    if standout is not None:
+        # one far key that every query must find: its score stands out by construction
+        b, t = standout
+        k, v = dense[b]
+        k[t] = k[t] * 0 + 1.0
+        v[t] = v[t] * 0 + 7.0
+        blk = int(table[slots[b], t // BS])
+        kc[blk, :, t % BS, :] = 1.0
+        vc[blk, :, :, t % BS] = 7.0
+        q = q * 0.01 + 3.0
+        q = q.to(dtype)
+    row_seq, row_pos, cu = [], [], [0]
+    for b, (n, m) in enumerate(zip(lengths, new)):
+        row_seq += [b] * m
+        row_pos += list(range(n - m, n))
+        cu.append(cu[-1] + m)
+    qd = q.to(DEV)
+    out = torch.empty_like(qd)
+    scale = 1.0 / math.sqrt(head_dim)
+    kn.force_generic = force_generic
+    try:
+        need = kn.attention_workspace(dtype, rows, heads, kv_heads, head_dim, BS, decode, max(lengths))
+        ws = torch.empty(need, dtype=torch.float32, device=DEV) if need else None
+        kn.attention(qd, out, heads, kv_heads, head_dim, i32(row_pos), i32(row_seq), i32(slots), i32(cu),
+                     table, kc, vc, BS, scale, window, decode=decode, max_len=max(lengths), workspace=ws)
+    finally:
+        kn.force_generic = False
+    want = torch.zeros((rows, heads, head_dim), dtype=torch.float64)
+    r = 0
+    for b, (n, m) in enumerate(zip(lengths, new)):
+        k, v = dense[b]
+        # plain attention over the whole sequence with the real queries in the last m places
+        qfull = torch.zeros((n, heads, head_dim), dtype=torch.float64)
+        qfull[n - m:] = q[r : r + m].double().view(m, heads, head_dim)
+        want[r : r + m] = plain.attention(qfull, k, v, window=window)[n - m:]
+        r += m
+    return out.view(rows, heads, head_dim), want
+
+
+@pytest.mark.parametrize("dtype,generic", [(torch.float32, True), (torch.bfloat16, True), (torch.bfloat16, False)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(4, 2, 64), (3, 1, 32), (6, 3, 48), (8, 8, 128), (2, 1, 96)])
+def test_attention_prompts(kn, dtype, generic, heads, kv_heads, head_dim):
+    got, want = run_attention(kn, None, [5, 70, 131, 1], [5, 70, 40, 1], heads, kv_heads, head_dim, dtype, 21,
+                              force_generic=generic)
+    assert rel_err(got, want) < (2e-6 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("dtype,generic", [(torch.float32, True), (torch.bfloat16, False)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(32, 8, 128), (3, 1, 32), (16, 1, 64), (6, 3, 48)])
+def test_attention_decoding_over_long_keys(kn, dtype, generic, heads, kv_heads, head_dim):
+    got, want = run_attention(kn, None, [700, 64, 257, 1, 300], [1, 1, 1, 1, 1], heads, kv_heads, head_dim,
+                              dtype, 22, decode=True, force_generic=generic)
+    assert rel_err(got, want) < (2e-6 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("dtype,generic", [(torch.float32, True), (torch.bfloat16, True), (torch.bfloat16, False)])
+@pytest.mark.parametrize("window", [1, 33, 64, 100])
+def test_attention_window_edge(kn, dtype, generic, window):
+    got, want = run_attention(kn, None, [150, 40], [150, 3], 4, 2, 64, dtype, 23, window=window, force_generic=generic)
+    assert rel_err(got, want) < (2e-6 if dtype == torch.float32 else 8e-3)
+    got, want = run_attention(kn, None, [300, 99], [1, 1], 4, 2, 64, dtype, 24, window=window, decode=True,
+                              force_generic=generic)
+    assert rel_err(got, want) < (2e-6 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("dtype,generic", [(torch.float32, True), (torch.bfloat16, False)])
+@pytest.mark.parametrize("decode", [False, True])
+def test_attention_finds_one_far_key_among_hundreds(kn, dtype, generic, decode):
+    """Key 3 of 600 carries score ~ 3 * hd / sqrt(hd) above the rest: the output must be its value."""
+    new = [1, 1] if decode else [17, 2]
+    got, want = run_attention(kn, None, [600, 130], new, 4, 2, 64, dtype, 25, decode=decode, force_generic=generic,
+                              standout=(0, 3))
+    assert rel_err(got, want) < (2e-6 if dtype == torch.float32 else 8e-3)
+    assert float((got[0].double().cpu() - 7.0).abs().max()) < 0.1
+
+
+def test_attention_reference_vectors(kn):
+    """q = k = v = 0.1 over 256 keys gives 0.1, 0.05 over 1500 keys gives 0.05
+    (internal/device/attention_test.go:10-94)."""
+    for n, val, heads in ((256, 0.1, 8), (1500, 0.05, 1)):
+        hd = 128
+        blocks = (n + BS - 1) // BS
+        kc = torch.full((blocks, heads, BS, hd), val, dtype=torch.float32, device=DEV)
+        vc = torch.full((blocks, heads, hd, BS), val, dtype=torch.float32, device=DEV)
+        table = torch.arange(blocks, dtype=torch.int32, device=DEV).view(1, -1)
+        q = torch.full((1, heads * hd), val, dtype=torch.float32, device=DEV)
+        out = torch.empty_like(q)
+        kn.attention(q, out, heads, heads, hd, i32([n - 1]), i32([0]), i32([0]), i32([0, 1]), table, kc, vc, BS,
+                     1 / math.sqrt(hd), 0, decode=True, max_len=n)
+        assert float((out - val).abs().max()) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_store_rotates_and_writes_the_right_rows(kn, dtype):
+    heads, kv_heads, hd = 6, 3, 48
+    freqs = plain.rope_frequencies(hd, 25000.0)
+    pos = [0, 5, 63, 64, 200]
+    rows = len(pos)
+    width = (heads + 2 * kv_heads) * hd
+    qkv = rnd((rows, width), 31, dtype)
+    orig = qkv.clone()
+    n_blocks = 6
+    kc = torch.zeros((n_blocks, kv_heads, BS, hd), dtype=dtype, device=DEV)
+    vc = torch.zeros((n_blocks, kv_heads, hd, BS), dtype=dtype, device=DEV)
+    table = torch.tensor([[0, 0, 0, 0], [5, 2, 4, 1]], dtype=torch.int32, device=DEV)  # slot 1 is used
+    q = qkv[:, : heads * hd]
+    k = qkv[:, heads * hd : (heads + kv_heads) * hd]
+    v = qkv[:, (heads + kv_heads) * hd :]
+    kn.rope_store(q, k, v, heads, kv_heads, hd, freqs.to(DEV), i32(pos), i32([0] * rows), i32([1]), table, kc, vc, BS)
+    tol = 2e-6 if dtype == torch.float32 else 5e-3
+    want_q = plain.rope(orig[:, : heads * hd].cpu().view(rows, heads, hd), pos, freqs)
+    assert rel_err(q.reshape(rows, heads, hd), want_q) < tol
+    want_k = plain.rope(orig[:, heads * hd : (heads + kv_heads) * hd].cpu().view(rows, kv_heads, hd), pos, freqs)
+    phys = [5, 2, 4, 1]
+    written = torch.zeros_like(kc, dtype=torch.bool)
+    for r, p in enumerate(pos):
+        blk, off = phys[p // BS], p % BS
+        assert rel_err(kc[blk, :, off, :], want_k[r]) < tol
+        assert torch.equal(vc[blk, :, :, off], orig[r, (heads + kv_heads) * hd :].view(kv_heads, hd))
+        written[blk, :, off, :] = True
+    # writing position p changes row p only (internal/device/kvcache_test.go:88-104)
+    assert float(kc[~written].abs().max()) == 0.0
+    # the reference's own vector: hd 128, 32 heads, pos 5, theta 1e4, input i/100
+    # (internal/device/rope_test.go:10-65)
+    x = (torch.arange(32 * 128, dtype=torch.float32) / 100.0).view(1, -1).to(dtype).to(DEV)
+    x0 = x.clone()
+    f = plain.rope_frequencies(128, 10000.0)
+    kn.rope_store(x, None, None, 32, 0, 128, f.to(DEV), i32([5]))
+    assert float((x.double().cpu().view(1, 32, 128) - plain.rope(x0.cpu().view(1, 32, 128), [5], f)).abs().max()) \
+        < (1e-4 if dtype == torch.float32 else 0.2)
