@@ -6,12 +6,13 @@ kernels.
 """
 from . import models  # noqa: F401  (registers the architectures)
 from .config import ConfigError, LlamaConfig, ModelConfig
-from .engine import Engine, StepEntry
+from .engine import Engine, GenerationResult, StepEntry, generate
 from .loading import load_engine, random_engine
+from .sampling import SamplingParams
 from .registry import register_architecture, registered_architectures
 from .weights import WeightError, write_model_folder
 
 __all__ = [
     "ConfigError", "LlamaConfig", "ModelConfig", "Engine", "StepEntry", "load_engine", "random_engine",
-    "register_architecture", "registered_architectures", "WeightError", "write_model_folder",
+    "GenerationResult", "generate", "SamplingParams", "register_architecture", "registered_architectures", "WeightError", "write_model_folder",
 ]

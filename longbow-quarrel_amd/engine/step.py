@@ -82,6 +82,8 @@ class Engine:
         self.meta = StepMeta(env.device)
         self.stream = torch.cuda.Stream(device=env.device) if env.device.type == "cuda" else None
         self.steps_run = 0
+        #: whether every part only launches library kernels (then decoding steps can be captured)
+        self.graph_safe = all(getattr(b, "graph_safe", False) for b in model.blocks)
 
     # ---- sequences ---------------------------------------------------------------------
     def new_sequence(self) -> int:
@@ -114,21 +116,26 @@ class Engine:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"slot {e.slot}: wanted place {w} is outside its {len(e.tokens)} tokens")
 
+    def run_on_stream(self, fn):
+        """Runs fn() with the engine's stream current, ordered after what the caller has queued and
+        before what it queues next."""
+        if self.stream is None:
+            return fn()
+        self.stream.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(self.stream):
+            self.kernels.use_stream(self.stream)
+            try:
+                out = fn()
+            finally:
+                self.kernels.use_stream(None)
+        torch.cuda.current_stream(self.device).wait_stream(self.stream)
+        return out
+
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Runs the entries' tokens; returns float32 logits [wanted, vocab] in the order of the
         entries and of each entry's `want` (None if nothing is wanted)."""
         self._validate(entries)
-        if self.stream is not None:
-            self.stream.wait_stream(torch.cuda.current_stream(self.device))
-            with torch.cuda.stream(self.stream):
-                self.kernels.use_stream(self.stream)
-                try:
-                    out = self._step(entries)
-                finally:
-                    self.kernels.use_stream(None)
-            torch.cuda.current_stream(self.device).wait_stream(self.stream)
-            return out
-        return self._step(entries)
+        return self.run_on_stream(lambda: self._step(entries))
 
     def _step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         cache = self.cache

@@ -288,3 +288,83 @@ class HipKernels:
             c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
             c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
             c_longlong(ws_n), c_int(1 if self.force_generic else 0), self.stream))
+
+    # ------------------------------------------------------------------ sampling
+    def apply_penalty(self, logits: torch.Tensor, seq_slot: torch.Tensor, recent: torch.Tensor,
+                      recent_n: torch.Tensor, penalty: float) -> None:
+        """Repetition penalty on the distinct ids in each sequence's ring of recent tokens, in place."""
+        self._dev(logits, seq_slot, recent, recent_n)
+        rows, vocab = logits.shape
+        self._i32(seq_slot, "seq_slot", rows)
+        if logits.dtype != torch.float32 or recent.dtype != torch.int32 or recent_n.dtype != torch.int32 \
+                or recent.dim() != 2 or recent.shape[1] != 64 or not recent.is_contiguous():
+            raise KernelLibraryError("penalty: logits float32, ring int32 [slots, 64], counters int32")
+        self._check(self.lib.lq_apply_penalty(_ptr(logits), c_int(self._rows2d(logits, "logits")), c_int(rows),
+                                              c_int(vocab), _ptr(seq_slot), _ptr(recent), _ptr(recent_n),
+                                              c_float(penalty), self.stream))
+
+    def argmax(self, logits: torch.Tensor, out: torch.Tensor, seq_slot: Optional[torch.Tensor] = None,
+               recent: Optional[torch.Tensor] = None, recent_n: Optional[torch.Tensor] = None) -> None:
+        """out[r] = first maximal index of logits[r]; the token is pushed into the ring if one is given."""
+        self._dev(logits, out, seq_slot, recent, recent_n)
+        rows, vocab = logits.shape
+        self._i32(out, "argmax out", rows)
+        if logits.dtype != torch.float32:
+            raise KernelLibraryError("argmax: logits must be float32")
+        if recent is not None:
+            self._i32(seq_slot, "seq_slot", rows)
+        self._check(self.lib.lq_argmax(_ptr(logits), c_int(self._rows2d(logits, "logits")), c_int(rows),
+                                       c_int(vocab), _ptr(seq_slot), _ptr(out), _ptr(recent), _ptr(recent_n),
+                                       self.stream))
+
+    def sample(self, logits: torch.Tensor, out: torch.Tensor, seq_slot: torch.Tensor, temperature: float,
+               top_k: int, top_p: float, rng_key: torch.Tensor, rng_ctr: torch.Tensor,
+               recent: Optional[torch.Tensor] = None, recent_n: Optional[torch.Tensor] = None,
+               kept_count: Optional[torch.Tensor] = None, kept_mass: Optional[torch.Tensor] = None) -> None:
+        """Temperature sampling with top-k and top-p; each sequence's counter moves on by one."""
+        self._dev(logits, out, seq_slot, rng_key, rng_ctr, recent, recent_n, kept_count, kept_mass)
+        rows, vocab = logits.shape
+        self._i32(out, "sample out", rows)
+        self._i32(seq_slot, "seq_slot", rows)
+        if logits.dtype != torch.float32 or rng_key.dtype != torch.int64 or rng_ctr.dtype != torch.int64:
+            raise KernelLibraryError("sample: logits float32, generator key and counter int64")
+        if kept_count is not None:
+            self._i32(kept_count, "kept_count", rows)
+        if kept_mass is not None and (kept_mass.dtype != torch.float64 or kept_mass.numel() < rows):
+            raise KernelLibraryError("sample: kept_mass must be float64 with one entry a row")
+        self._check(self.lib.lq_sample(_ptr(logits), c_int(self._rows2d(logits, "logits")), c_int(rows),
+                                       c_int(vocab), _ptr(seq_slot), c_float(temperature), c_int(top_k),
+                                       c_float(top_p), _ptr(rng_key), _ptr(rng_ctr), _ptr(recent), _ptr(recent_n),
+                                       _ptr(out), _ptr(kept_count), _ptr(kept_mass), self.stream))
+
+    def advance(self, row_pos: torch.Tensor, seq_start: torch.Tensor, seq_len: torch.Tensor, batch: int) -> None:
+        """Positions and lengths of a decoding batch move on by one."""
+        self._dev(row_pos, seq_start, seq_len)
+        for t in (row_pos, seq_start, seq_len):
+            self._i32(t, "advance", batch)
+        self._check(self.lib.lq_advance(_ptr(row_pos), _ptr(seq_start), _ptr(seq_len), c_int(batch), self.stream))
+
+    def record(self, tokens: torch.Tensor, history: torch.Tensor, step_index: torch.Tensor, batch: int) -> None:
+        """history[step_index] = tokens; step_index += 1 (nothing is written past the last row)."""
+        self._dev(tokens, history, step_index)
+        self._i32(tokens, "record tokens", batch)
+        if history.dtype != torch.int32 or history.dim() != 2 or history.shape[1] != batch or not history.is_contiguous():
+            raise KernelLibraryError("record: history must be dense int32 [steps, batch]")
+        self._i32(step_index, "step_index", 1)
+        self._check(self.lib.lq_record(_ptr(tokens), _ptr(history), c_int(batch), _ptr(step_index),
+                                       c_int(history.shape[0]), self.stream))
+
+    # ------------------------------------------------------------------ HIP graphs
+    def graph_begin(self) -> None:
+        self._check(self.lib.lq_graph_begin(self.stream))
+
+    def graph_end(self) -> int:
+        handle = c_void_p(0)
+        self._check(self.lib.lq_graph_end(self.stream, ctypes.byref(handle)))
+        return int(handle.value)
+
+    def graph_launch(self, handle: int) -> None:
+        self._check(self.lib.lq_graph_launch(c_void_p(handle), self.stream))
+
+    def graph_destroy(self, handle: int) -> None:
+        self._check(self.lib.lq_graph_destroy(c_void_p(handle)))

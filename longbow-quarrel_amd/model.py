@@ -113,6 +113,8 @@ class DecoderModel:
         picked = ctx.ws.alloc((n_want, s.width), torch.float32)
         kn.gather_rows(x, want_rows, picked, delta=pending)
         normed = self.final_norm.forward(picked, ctx)
-        logits = torch.empty((n_want, s.vocab_size), dtype=torch.float32, device=ctx.device)
+        logits = ctx.logits_out
+        if logits is None:
+            logits = torch.empty((n_want, s.vocab_size), dtype=torch.float32, device=ctx.device)
         project(kn, ctx, normed, self.head, logits)
         return logits

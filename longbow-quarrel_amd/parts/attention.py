@@ -23,6 +23,10 @@ from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mix
 
 @MIXERS.register("gqa_attention")
 class GQAttention(Mixer):
+    @property
+    def graph_safe(self) -> bool:
+        return self.position.graph_safe
+
     def __init__(self, width: int, heads: int, kv_heads: int, head_dim: int, position: PartSpec,
                  prefix: str, scale: Optional[float] = None, window: int = 0,
                  names: Optional[Mapping[str, str]] = None) -> None:

@@ -185,6 +185,7 @@ class StepContext:
     max_new: int = 0
     max_len: int = 0
     decode: bool = False  # every sequence brings exactly one token
+    logits_out: Optional[torch.Tensor] = None  # where the logits go (a captured step's fixed buffer)
 
 
 @dataclass
@@ -206,6 +207,11 @@ class LayerCache:
 
 class Part:
     """Declares the tensors it binds; receives them in `bind`."""
+
+    #: True if forward() does nothing but launch the library's kernels on buffers from ctx.ws:
+    #: no allocation, no host synchronisation, no other library's operators.  Only then may a
+    #: step that contains the part be captured into a HIP graph.
+    graph_safe = False
 
     def tensor_specs(self) -> List[TensorSpec]:
         return []

@@ -20,6 +20,10 @@ class PreNormBlock(Block):
         self.mixer_norm = build_part(NORMS, mixer_norm)
         self.ffn_norm = build_part(NORMS, ffn_norm)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in self.parts())
+
     def parts(self):
         return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
 

@@ -13,6 +13,8 @@ from .base import FEED_FORWARDS, BuildEnv, FeedForward, StepContext, TensorSpec,
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, width: int, inner: int, prefix: str, names: Optional[Mapping[str, str]] = None) -> None:
         self.width, self.inner = int(width), int(inner)
         n = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}

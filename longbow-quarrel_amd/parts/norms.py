@@ -13,6 +13,8 @@ from .base import NORMS, VECTOR32, BuildEnv, Norm, StepContext, TensorSpec
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, width: int, eps: float, name: str) -> None:
         self.width = int(width)
         self.eps = float(eps)

@@ -43,6 +43,8 @@ def rotary_frequencies(head_dim: int, base: float, scaling: Optional[Mapping] = 
 
 @POSITION_ENCODINGS.register("rope")
 class RotaryEncoding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, head_dim: int, base: float, scaling: Optional[Mapping] = None) -> None:
         self.head_dim = int(head_dim)
         self.base = float(base)
@@ -62,6 +64,8 @@ class RotaryEncoding(PositionEncoding):
 
 @POSITION_ENCODINGS.register("none")
 class NoPositionEncoding(PositionEncoding):
+    graph_safe = True
+
     """Leaves q and k as they are (the mixer sees order through the causal mask only)."""
 
     def __init__(self, **_unused) -> None:

@@ -1,0 +1,33 @@
+"""Picks the next token of every sequence of a batch from its logits, on the device."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .params import SamplingParams
+from .state import SamplerState
+
+
+class NonFiniteLogits(RuntimeError):
+    """The reference falls back to the first finite index (internal/engine/sampler.go:73-75,
+    107-123); a library that is checked for exactness reports the fault instead."""
+
+
+class Sampler:
+    def __init__(self, kernels, state: SamplerState, params: SamplingParams) -> None:
+        self.kernels = kernels
+        self.state = state
+        self.params = params
+
+    def sample(self, logits: torch.Tensor, seq_slot: torch.Tensor, out: torch.Tensor) -> None:
+        """logits float32 [batch, vocab] (changed in place by the penalty), seq_slot int32 [batch],
+        out int32 [batch].  Launches only; safe inside a graph capture."""
+        p, st, kn = self.params, self.state, self.kernels
+        if p.repetition_penalty > 1.0:
+            kn.apply_penalty(logits, seq_slot, st.recent, st.recent_n, p.repetition_penalty)
+        if p.greedy:
+            kn.argmax(logits, out, seq_slot, st.recent, st.recent_n)
+        else:
+            kn.sample(logits, out, seq_slot, p.temperature, p.top_k, p.top_p, st.rng_key, st.rng_ctr,
+                      st.recent, st.recent_n)
