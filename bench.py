@@ -1,0 +1,172 @@
+"""Decode and prefill throughput of the Llama 3 8B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Default run: the 8B layer sizes with random bfloat16 weights, a batch of 8
+sequences that start from 512-token random prompts; W untimed decode steps, then
+exactly K timed ones (a step = one token for every sequence of the batch: model,
+greedy sampling on the device and state upkeep, replayed as a HIP graph, tokens read
+back by the host every step as generation does).  `value` is decoded tokens a
+second.  The same line carries a 2,048-token prefill, the decode step's HBM
+roofline, and decode at batch 1 and 64.  One JSON line on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_GBPS = 8000.0  # MI355X published peak
+BF16_TFLOPS = 2500.0  # dense MFMA bf16
+
+CONFIG_8B = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "intermediate_size": 14336,
+    "num_hidden_layers": 32, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "vocab_size": 128256, "max_position_embeddings": 8192, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": None, "tie_word_embeddings": False, "torch_dtype": "bfloat16",
+    "bos_token_id": 128000, "eos_token_id": 128001,
+}
+
+
+def weight_bytes_per_step(c) -> float:
+    """Every weight a decode step uses, once: the layers' matrices and norms, the final norm and the head
+    (of the embedding table only the batch's rows are read)."""
+    d, i, hd = c.hidden_size, c.intermediate_size, c.head_dim
+    nh, nkv = c.num_attention_heads, c.num_key_value_heads
+    per_layer = 2 * (d * (nh + 2 * nkv) * hd + nh * hd * d + 3 * d * i) + 4 * 2 * d
+    return c.num_hidden_layers * per_layer + 2 * c.vocab_size * d + 4 * d
+
+
+def kv_bytes_per_token(c) -> float:
+    return 2 * c.num_key_value_heads * c.head_dim * 2 * c.num_hidden_layers
+
+
+def prefill_flops(c, t: int) -> float:
+    d, i, hd = c.hidden_size, c.intermediate_size, c.head_dim
+    nh, nkv = c.num_attention_heads, c.num_key_value_heads
+    linear = 2.0 * t * (d * (nh + 2 * nkv) * hd + nh * hd * d + 3 * d * i)
+    attention = 2.0 * 2.0 * nh * hd * t * (t + 1) / 2.0  # causal: scores and values
+    return c.num_hidden_layers * (linear + attention) + 2.0 * d * c.vocab_size
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the 8B shape has (0 = all 32)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--no-points", action="store_true", help="skip the prefill and the batch 1 / 64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    import longbow_quarrel_amd as lq
+    from longbow_quarrel_amd.engine import EngineBackend, StepEntry
+
+    cfg = dict(CONFIG_8B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    config = lq.LlamaConfig.from_dict(cfg)
+    slot_len = cfg["max_position_embeddings"]
+    max_batch = 64 if not args.no_points else args.batch
+    t0 = time.time()
+    engine = lq.random_engine(config, seed=0, dtype="bfloat16", max_tokens=max_batch * slot_len, max_slots=max_batch)
+    torch.cuda.synchronize()
+    print(f"[bench] model and cache ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+    gen = torch.Generator().manual_seed(1234)
+
+    def random_prompt(n: int):
+        return torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
+
+    def decode_run(batch: int, prompt_len: int, steps: int, warmup: int):
+        """tokens a second, ms a step, mean context during the timed steps"""
+        backend = EngineBackend(engine, lq.SamplingParams(temperature=0.0), use_graphs=True)
+        slots = [backend.new_sequence(r, [0]) for r in range(batch)]
+        prompts = [random_prompt(prompt_len) for _ in range(batch)]
+        # prompts in chunks of sequences so that a prefill step stays at a few thousand rows
+        toks = []
+        per = max(1, 4096 // prompt_len)
+        for i in range(0, batch, per):
+            toks += backend.prefill(slots[i : i + per], prompts[i : i + per])
+        for _ in range(warmup):
+            toks = backend.decode(slots, toks, False)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            toks = backend.decode(slots, toks, False)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        ctx_mean = prompt_len + warmup + (steps + 1) / 2.0
+        for s in slots:
+            backend.release(s)
+        backend.close()
+        return batch * steps / dt, dt / steps * 1e3, ctx_mean
+
+    value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
+    step_bytes = weight_bytes_per_step(config) + args.batch * ctx_mean * kv_bytes_per_token(config)
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
+
+    prefill = None
+    points = {}
+    if not args.no_points:
+        t_tokens = 2048
+        slot = engine.new_sequence()
+        prompt = random_prompt(t_tokens)
+        # once untimed (first launches), then timed on a fresh slot
+        engine.step([StepEntry(slot, prompt, [t_tokens - 1])])
+        engine.release(slot)
+        slot = engine.new_sequence()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        engine.step([StepEntry(slot, prompt, [t_tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        engine.release(slot)
+        prefill = {
+            "value": round(t_tokens / dt, 1), "tokens": t_tokens, "ms": round(dt * 1e3, 3),
+            "frac": round(prefill_flops(config, t_tokens) / dt / (BF16_TFLOPS * 1e12), 4),
+        }
+        print(f"[bench] prefill: {prefill}", file=sys.stderr, flush=True)
+        v1, _, _ = decode_run(1, args.prompt_len, max(16, args.steps // 2), max(4, args.warmup // 2))
+        v64, _, _ = decode_run(64, args.prompt_len, max(16, args.steps // 4), max(4, args.warmup // 2))
+        points = {"decode_b1": round(v1, 1), "decode_b64": round(v64, 1)}
+        print(f"[bench] points: {points}", file=sys.stderr, flush=True)
+
+    line = {
+        "metric": "decode tok/s (Llama-3 8B shape, bf16, batch 8, 512-token prompts)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic: random weights N(0, 0.02) from a seed, uniform random token ids",
+        "config": {
+            "model": "llama3-8b-shape", "layers": config.num_hidden_layers, "layers_full": full_layers,
+            "hidden": config.hidden_size, "heads": config.num_attention_heads,
+            "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+            "intermediate": config.intermediate_size, "vocab": config.vocab_size,
+            "rope_theta": config.rope_theta, "rms_eps": config.rms_norm_eps, "tied": config.tie_word_embeddings,
+            "global_batch": args.batch, "seq_len": args.prompt_len, "context": slot_len,
+            "new_tokens": args.steps + args.warmup, "sampling": "greedy", "parallelism": "single-gpu",
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -31,7 +31,7 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr int BS = 64;      // positions per cache block (the only block size this file takes)
-constexpr int SPLIT = 256;  // keys per split when decoding
+constexpr int SPLIT = 128;  // keys per split when decoding
 
 __device__ inline bf16x8 as_bf16x8(u32x4 v) {
   union {
@@ -72,24 +72,56 @@ struct AttnArgs {
 // p_c, its first key lo_c.  Keys t_begin..t_end (inclusive) are walked; t_begin is a multiple of 32.
 // On return o[dt][e] holds the unnormalised O^T[dt*16 + (lane/16)*4 + e][c], m the running maximum
 // (in the log2 domain) and l this lane's share of the normaliser (to be summed over lane/16).
+// One chunk's operands as they come from memory: 16 bytes a lane for each K fragment, two 8-byte
+// pieces a lane for each V^T fragment.
+template <int HD>
+struct ChunkRegs {
+  u32x4 k[2][HD / 32];
+  u32x2 v[HD / 16][2];
+};
+
+template <int HD>
+__device__ inline void load_chunk(const AttnArgs& a, int kvh, long long blk, int koff, ChunkRegs<HD>& r) {
+  const int lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
+  const bf16_t* kb = a.kcache + ((blk * a.nkv + kvh) * BS + koff) * (long long)HD;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int kk = 0; kk < HD / 32; ++kk)
+      r.k[j][kk] = *(const u32x4*)(kb + (16 * j + c16) * HD + kk * 32 + g * 8);
+  const bf16_t* vb = a.vcache + ((blk * a.nkv + kvh) * (long long)HD) * BS + koff;
+#pragma unroll
+  for (int dt = 0; dt < HD / 16; ++dt) {
+    const bf16_t* vr = vb + (long long)(dt * 16 + c16) * BS;
+    r.v[dt][0] = *(const u32x2*)(vr + g * 4);
+    r.v[dt][1] = *(const u32x2*)(vr + 16 + g * 4);
+  }
+}
+
 template <int HD>
 __device__ inline void attend(const AttnArgs& a, const bf16x8 (&qf)[HD / 32], int kvh, const int* table,
                               int t_begin, int t_end, bool col_valid, int p_c, int lo_c,
                               f32x4 (&o)[HD / 16], float& m, float& l) {
-  const int lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
+  const int lane = threadIdx.x & 63, g = lane >> 4;
+  // the next chunk's keys and values are already on their way while this chunk is computed, and
+  // the block number of the chunk after that while those are loaded
+  ChunkRegs<HD> cur, nxt;
+  long long blk_next = table[t_begin / BS];
+  load_chunk<HD>(a, kvh, blk_next, t_begin % BS, nxt);
+  blk_next = (t_begin + 32 <= t_end) ? table[(t_begin + 32) / BS] : 0;
   for (int t0 = t_begin; t0 <= t_end; t0 += 32) {
-    const long long blk = table[t0 / BS];
-    const int koff = t0 % BS;
-    const bf16_t* kb = a.kcache + ((blk * a.nkv + kvh) * BS + koff) * (long long)HD;
+    cur = nxt;
+    if (t0 + 32 <= t_end) {
+      load_chunk<HD>(a, kvh, blk_next, (t0 + 32) % BS, nxt);
+      blk_next = (t0 + 64 <= t_end) ? table[(t0 + 64) / BS] : 0;
+    }
     f32x4 s[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       s[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < HD / 32; ++kk) {
-        const u32x4 kv = *(const u32x4*)(kb + (16 * j + c16) * HD + kk * 32 + g * 8);
-        s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kv), qf[kk], s[j], 0, 0, 0);
-      }
+      for (int kk = 0; kk < HD / 32; ++kk)
+        s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.k[j][kk]), qf[kk], s[j], 0, 0, 0);
     }
     float sv[8];
     float cmax = -INFINITY;
@@ -126,12 +158,10 @@ __device__ inline void attend(const AttnArgs& a, const bf16x8 (&qf)[HD / 32], in
     // keys past t_end lie in the block but were never written: their values must not reach the
     // product (0 * garbage may be NaN), so they are zeroed
     const bool tail = t0 + 31 > t_end;
-    const bf16_t* vb = a.vcache + ((blk * a.nkv + kvh) * (long long)HD) * BS + koff;
 #pragma unroll
     for (int dt = 0; dt < HD / 16; ++dt) {
-      const bf16_t* vr = vb + (long long)(dt * 16 + c16) * BS;
-      u32x2 v0 = *(const u32x2*)(vr + g * 4);
-      u32x2 v1 = *(const u32x2*)(vr + 16 + g * 4);
+      u32x2 v0 = cur.v[dt][0];
+      u32x2 v1 = cur.v[dt][1];
       if (tail) {
         const int ta = t0 + g * 4, tb = t0 + 16 + g * 4;
         if (ta + 0 > t_end) v0[0] &= 0xffff0000u;

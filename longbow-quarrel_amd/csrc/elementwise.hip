@@ -55,13 +55,87 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ del
   }
 }
 
+// The same, for rows that fit the block's registers: width a multiple of 4 and at most
+// 256 threads * NV * 4.  One read of x (and delta), one write of each output.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ inline f32x4_t load4(const float* p) { return *(const f32x4_t*)p; }
+__device__ inline f32x4_t load4(const bf16_t* p) {
+  const u32x2_t r = *(const u32x2_t*)p;
+  f32x4_t v;
+  v[0] = __uint_as_float(r[0] << 16);
+  v[1] = __uint_as_float(r[0] & 0xffff0000u);
+  v[2] = __uint_as_float(r[1] << 16);
+  v[3] = __uint_as_float(r[1] & 0xffff0000u);
+  return v;
+}
+__device__ inline void store4(float* p, f32x4_t v) { *(f32x4_t*)p = v; }
+__device__ inline void store4(bf16_t* p, f32x4_t v) {
+  u32x2_t r;
+  r[0] = (unsigned)f32_to_bf16(v[0]).bits | ((unsigned)f32_to_bf16(v[1]).bits << 16);
+  r[1] = (unsigned)f32_to_bf16(v[2]).bits | ((unsigned)f32_to_bf16(v[3]).bits << 16);
+  *(u32x2_t*)p = r;
+}
+
+template <typename TD, typename TO, bool HAS_DELTA, int NV>
+__global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                                           const float* __restrict__ w, TO* __restrict__ out,
+                                                           int D, float eps) {
+  __shared__ float red[16];
+  const long long base = (long long)blockIdx.x * D;
+  f32x4_t v[NV];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int j = (threadIdx.x + i * 256) * 4;
+    if (j < D) {
+      v[i] = load4(x + base + j);
+      if (HAS_DELTA) {
+        v[i] += load4(delta + base + j);
+        store4(x + base + j, v[i]);
+      }
+      ss += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int j = (threadIdx.x + i * 256) * 4;
+    if (j < D) store4(out + base + j, v[i] * r * load4(w + j));
+  }
+}
+
+template <typename TD, typename TO, bool HAS>
+static void rmsnorm_launch(float* x, const void* delta, const float* w, void* out, int rows, int D, float eps,
+                           hipStream_t stream) {
+  const bool aligned = D % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                       ((uintptr_t)w % 16) == 0 && ((uintptr_t)delta % 16) == 0;
+  const int vecs = (D / 4 + 255) / 256;
+  if (aligned && vecs <= 8) {
+#define LQ_REGS(NV) \
+  rmsnorm_regs_kernel<TD, TO, HAS, NV><<<rows, 256, 0, stream>>>(x, (const TD*)delta, w, (TO*)out, D, eps)
+    if (vecs <= 1)
+      LQ_REGS(1);
+    else if (vecs <= 2)
+      LQ_REGS(2);
+    else if (vecs <= 4)
+      LQ_REGS(4);
+    else
+      LQ_REGS(8);
+#undef LQ_REGS
+    return;
+  }
+  const int threads = D >= 2048 ? 512 : (D >= 512 ? 256 : 64);
+  rmsnorm_kernel<TD, TO, HAS><<<rows, threads, 0, stream>>>(x, (const TD*)delta, w, (TO*)out, D, eps);
+}
+
 extern "C" int lq_rmsnorm(float* x, const void* delta, int delta_dtype, const float* w, float eps,
                           void* out, int out_dtype, int rows, int D, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && D > 0, "rmsnorm: rows %d and width %d must be positive", rows, D);
   LQ_REQUIRE(out_dtype == LQ_F32 || out_dtype == LQ_BF16, "rmsnorm: unknown out dtype %d", out_dtype);
-  const int threads = D >= 2048 ? 512 : (D >= 512 ? 256 : 64);
-#define LQ_NORM_LAUNCH(TD, TO, HAS)                                                         \
-  rmsnorm_kernel<TD, TO, HAS><<<rows, threads, 0, stream>>>(x, (const TD*)delta, w, (TO*)out, D, eps)
+#define LQ_NORM_LAUNCH(TD, TO, HAS) rmsnorm_launch<TD, TO, HAS>(x, delta, w, out, rows, D, eps, stream)
   if (delta == nullptr) {
     if (out_dtype == LQ_F32)
       LQ_NORM_LAUNCH(float, float, false);
@@ -200,8 +274,8 @@ extern "C" int lq_gather_rows(const float* x, const void* delta, int delta_dtype
 
 // ---------------------------------------------------------------- rotation + cache write
 // One block per row.  The row's position p comes from row_pos; its angles
-// p * f_i are formed in double from the double table f (hd/2 entries), so the
-// rotation is exact to 32-bit rounding at any position.  Pair (i, i + hd/2):
+// p * f_i are formed and reduced modulo 2 pi in double from the double table f
+// (hd/2 entries), so the rotation is exact to 32-bit rounding at any position.  Pair (i, i + hd/2):
 //   x_i' = x_i cos - x_{i+hd/2} sin ; x_{i+hd/2}' = x_i sin + x_{i+hd/2} cos
 // (internal/device/kernels.metal:430-463).  q is rotated in place; rotated k
 // and plain v go to the paged cache (internal/device/kernels.metal:1736-1749
@@ -223,10 +297,15 @@ __global__ void rope_store_kernel(T* __restrict__ q, const T* __restrict__ k, co
   const int p = row_pos[r];
   if (has_rope) {
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
-      double s, c;
-      sincos((double)p * freqs[i], &s, &c);
-      cs[i] = (float)c;
-      cs[half + i] = (float)s;
+      // angle and its reduction to [-pi, pi] in double, sine and cosine of the remainder in 32-bit
+      const double a = (double)p * freqs[i];
+      const double n = rint(a * 0.15915494309189533577);
+      double r = fma(-n, 6.283185307179586232, a);
+      r = fma(-n, 2.4492935982947064e-16, r);
+      float sn, c;
+      sincosf((float)r, &sn, &c);
+      cs[i] = c;
+      cs[half + i] = sn;
     }
   } else {
     for (int i = threadIdx.x; i < half; i += blockDim.x) {

@@ -5,7 +5,7 @@ int lq_gemm_generic(const void* x, const void* w, void* out, int in_dtype, int o
                     int N, int K, int lda, int ldw, int ldc, hipStream_t stream);
 bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int lda, int ldw);
 int lq_gemm_mfma(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K, int lda,
-                 int ldw, int ldc, hipStream_t stream);
+                 int ldw, int ldc, int epilogue, hipStream_t stream);
 
 extern "C" int lq_linear(const void* x, const void* w, void* out, int in_dtype, int out_dtype,
                          int M, int N, int K, int lda, int ldw, int ldc, int force_generic,
@@ -14,6 +14,23 @@ extern "C" int lq_linear(const void* x, const void* w, void* out, int in_dtype, 
   LQ_REQUIRE(lda >= K && ldw >= K && ldc >= N, "linear: a row stride is smaller than its row");
   LQ_REQUIRE(x && w && out, "linear: null pointer");
   if (!force_generic && lq_gemm_mfma_accepts(x, w, in_dtype, K, lda, ldw))
-    return lq_gemm_mfma(x, w, out, out_dtype, M, N, K, lda, ldw, ldc, stream);
+    return lq_gemm_mfma(x, w, out, out_dtype, M, N, K, lda, ldw, ldc, 0, stream);
   return lq_gemm_generic(x, w, out, in_dtype, out_dtype, M, N, K, lda, ldw, ldc, stream);
+}
+
+// Whether lq_linear_swiglu takes this problem (else: lq_linear into [M, 2I] and lq_swiglu).
+extern "C" int lq_linear_swiglu_supported(int in_dtype, int N, int K) {
+  return in_dtype == LQ_BF16 && N % 16 == 0 && K % 8 == 0;
+}
+
+// out[M, N/2] = silu(gate) * up where [gate | up] = x . W^T and W's N rows hold gate and up rows
+// interleaved in groups of 8 (rows 16j..16j+7 gate 8j..8j+7, rows 16j+8..16j+15 up 8j..8j+7).
+extern "C" int lq_linear_swiglu(const void* x, const void* w, void* out, int in_dtype, int out_dtype, int M,
+                                int N, int K, int lda, int ldw, int ldc, hipStream_t stream) {
+  LQ_REQUIRE(M > 0 && N > 0 && K > 0, "linear+swiglu: sizes M=%d N=%d K=%d must be positive", M, N, K);
+  LQ_REQUIRE(lda >= K && ldw >= K && ldc >= N / 2, "linear+swiglu: a row stride is smaller than its row");
+  LQ_REQUIRE(x && w && out, "linear+swiglu: null pointer");
+  LQ_REQUIRE(lq_linear_swiglu_supported(in_dtype, N, K) && lq_gemm_mfma_accepts(x, w, in_dtype, K, lda, ldw),
+             "linear+swiglu: needs bfloat16, 16-byte aligned rows, K %% 8 == 0 and N %% 16 == 0");
+  return lq_gemm_mfma(x, w, out, out_dtype, M, N, K, lda, ldw, ldc, 1, stream);
 }

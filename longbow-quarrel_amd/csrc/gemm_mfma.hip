@@ -48,11 +48,19 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
   *p = f32_to_bf16(v);
 }
 
+// Epilogues.  EPI_SWIGLU expects the weight rows interleaved in groups of 8: rows 16j..16j+7 are
+// gate rows 8j..8j+7 and rows 16j+8..16j+15 the matching up rows, so that the lane holding gate
+// column c (c % 16 < 8) finds its up value 8 lanes further; it writes silu(gate) * up to
+// out[m][8j + c % 8], an [M, N / 2] matrix.
+enum { EPI_NONE = 0, EPI_SWIGLU = 1 };
+
+__device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
 // ------------------------------------------------------------------ tiled
 constexpr int TBK = 64;           // k per stage
 constexpr int TLD = TBK + 8;      // padded LDS row, in elements (144 bytes: conflict-free b128 reads)
 
-template <int WM, int WN, typename TO>
+template <int WM, int WN, int EPI, typename TO>
 __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A, int lda,
                                                               const bf16_t* __restrict__ W, int ldw,
                                                               TO* __restrict__ C, int ldc, int M, int N,
@@ -145,24 +153,30 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
 #pragma unroll
     for (int j = 0; j < WN; ++j) {
       const int col = n0 + wn * WN * 32 + j * 32 + (lane & 31);
-      if (col >= N) continue;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int row = m0 + wm * WM * 32 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row < M) store_out<TO>(C + (long long)row * ldc + col, acc[i][j][e]);
+        if (EPI == EPI_SWIGLU) {
+          // gate column c (c % 16 < 8) and its up column c + 8 sit 8 lanes apart
+          const float up = __shfl(acc[i][j][e], lane + 8, 64);
+          if ((col & 15) < 8 && row < M && col + 8 < N)
+            store_out<TO>(C + (long long)row * ldc + ((col >> 4) << 3) + (col & 7), silu_mul(acc[i][j][e], up));
+        } else {
+          if (row < M && col < N) store_out<TO>(C + (long long)row * ldc + col, acc[i][j][e]);
+        }
       }
     }
 }
 
-template <int WM, int WN, typename TO>
+template <int WM, int WN, int EPI, typename TO>
 int launch_tiled(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                  hipStream_t stream) {
   constexpr int BM = 2 * WM * 32, BN = 2 * WN * 32;
   const int tiles_m = lq_ceil_div(M, BM), tiles_n = lq_ceil_div(N, BN);
   const size_t smem = (size_t)(BM + BN) * TLD * sizeof(uint16_t);
-  auto kernel = gemm_bf16_tiled_kernel<WM, WN, TO>;
+  auto kernel = gemm_bf16_tiled_kernel<WM, WN, EPI, TO>;
   static bool configured = false;
-  if (!configured) {
+  if (!configured && smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem);
     if (e != hipSuccess) {
@@ -179,84 +193,111 @@ int launch_tiled(const void* A, const void* W, void* C, int M, int N, int K, int
   return 0;
 }
 
-// ------------------------------------------------------------------ skinny (M <= 16)
-constexpr int SK_UNROLL = 4;  // 64-k chunks a wave keeps in flight (8 weight loads of 1 KiB)
+// ------------------------------------------------------------------ skinny (M <= 64)
+// 64-k chunks a wave keeps in flight (two weight loads of 1 KiB each): fewer when more row tiles
+// need their own x operands in registers
+constexpr int sk_unroll(int mt) { return mt == 1 ? 4 : 2; }
 
-template <int KW, typename TO>
+template <int KW, int MT, int EPI, typename TO>
 __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X, int ldx,
                                                                    const bf16_t* __restrict__ W, int ldw,
                                                                    TO* __restrict__ C, int ldc, int M,
                                                                    int N, int K) {
-  __shared__ float red[KW][256];
+  constexpr int SK_UNROLL = sk_unroll(MT);
+  __shared__ float red[KW][MT * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n0 = blockIdx.x * 16;
   const int g = lane >> 4;
   const int nrow = min(n0 + (lane & 15), N - 1);
-  const int mrow = min(lane & 15, M - 1);
   const bf16_t* wp = W + (long long)nrow * ldw + g * 8;
-  const bf16_t* xp = X + (long long)mrow * ldx + g * 8;
+  const bf16_t* xp[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) xp[t] = X + (long long)min(t * 16 + (lane & 15), M - 1) * ldx + g * 8;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
   // wave w takes 64-k chunks w, w + KW, w + 2 KW, ... : the block reads KW * 128 bytes of every
   // weight row at a time
   for (int kc = wave * 64; kc < K; kc += KW * 64 * SK_UNROLL) {
-    u32x4 wv[SK_UNROLL][2], xv[SK_UNROLL][2];
+    u32x4 wv[SK_UNROLL][2], xv[SK_UNROLL][MT][2];
 #pragma unroll
     for (int u = 0; u < SK_UNROLL; ++u) {
       const int k = kc + u * KW * 64;
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const bool ok = k + h * 32 + g * 8 < K;
-        wv[u][h] = ok ? __builtin_nontemporal_load((const u32x4*)(wp + k + h * 32)) : zero;
-        xv[u][h] = ok ? *(const u32x4*)(xp + k + h * 32) : zero;
+        wv[u][h] = ok ? *(const u32x4*)(wp + k + h * 32) : zero;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) xv[u][t][h] = ok ? *(const u32x4*)(xp[t] + k + h * 32) : zero;
       }
     }
 #pragma unroll
     for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
       for (int h = 0; h < 2; ++h)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[u][h]), as_bf16x8(wv[u][h]), acc, 0, 0, 0);
-  }
-  // acc[e] = C[(lane / 16) * 4 + e][n0 + lane % 16], partial over this wave's k
 #pragma unroll
-  for (int e = 0; e < 4; ++e) red[wave][e * 64 + lane] = acc[e];
+        for (int t = 0; t < MT; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[u][t][h]), as_bf16x8(wv[u][h]), acc[t],
+                                                           0, 0, 0);
+  }
+  // acc[t][e] = C[t * 16 + (lane / 16) * 4 + e][n0 + lane % 16], partial over this wave's k
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][t * 256 + e * 64 + lane] = acc[t][e];
   __syncthreads();
   if (wave == 0) {
-    const int col = n0 + (lane & 15);
+    const int c16 = lane & 15;
+    const int col = n0 + c16;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float s = 0.f;
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int w = 0; w < KW; ++w) s += red[w][e * 64 + lane];
-      const int row = g * 4 + e;
-      if (row < M && col < N) store_out<TO>(C + (long long)row * ldc + col, s);
-    }
+      for (int e = 0; e < 4; ++e) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < KW; ++w) s += red[w][t * 256 + e * 64 + lane];
+        const int row = t * 16 + g * 4 + e;
+        if (EPI == EPI_SWIGLU) {
+          const float up = __shfl(s, lane + 8, 64);
+          if (c16 < 8 && row < M && col + 8 < N) store_out<TO>(C + (long long)row * ldc + (n0 >> 1) + c16, silu_mul(s, up));
+        } else {
+          if (row < M && col < N) store_out<TO>(C + (long long)row * ldc + col, s);
+        }
+      }
   }
 }
 
-template <int KW, typename TO>
+template <int KW, int MT, int EPI, typename TO>
 int launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc,
                   hipStream_t stream) {
-  gemm_bf16_skinny_kernel<KW, TO><<<lq_ceil_div(N, 16), KW * 64, 0, stream>>>(
+  gemm_bf16_skinny_kernel<KW, MT, EPI, TO><<<lq_ceil_div(N, 16), KW * 64, 0, stream>>>(
       (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K);
   LQ_CHECK_LAUNCH("linear(mfma skinny)");
   return 0;
 }
 
-template <typename TO>
+template <int MT, int EPI, typename TO>
+int pick_skinny(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
+                hipStream_t stream) {
+  // enough waves to keep the memory system busy: about 8 a CU
+  const long long tiles = lq_ceil_div(N, 16);
+  const int chunks = lq_ceil_div(K, 64);
+  if (tiles * 4 >= 2048 || chunks < 8)
+    return launch_skinny<4, MT, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  if (tiles * 8 >= 2048 || chunks < 16 || MT > 2)
+    return launch_skinny<8, MT, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  return launch_skinny<16, MT, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+}
+
+template <int EPI, typename TO>
 int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
              hipStream_t stream) {
-  if (M <= 16) {
-    // enough waves to keep the memory system busy: about 8 a CU
-    const long long tiles = lq_ceil_div(N, 16);
-    const int chunks = lq_ceil_div(K, 64);
-    if (tiles * 4 >= 2048 || chunks < 8) return launch_skinny<4, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-    if (tiles * 8 >= 2048 || chunks < 16) return launch_skinny<8, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-    return launch_skinny<16, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-  }
-  if (M <= 64) return launch_tiled<1, 2, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-  return launch_tiled<2, 2, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  if (M <= 16) return pick_skinny<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  if (M <= 32) return pick_skinny<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  if (M <= 64) return pick_skinny<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  return launch_tiled<2, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
 }
 
 }  // namespace
@@ -268,9 +309,18 @@ bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int
 }
 
 int lq_gemm_mfma(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K, int lda,
-                 int ldw, int ldc, hipStream_t stream) {
-  if (out_dtype == LQ_F32) return dispatch<float>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-  if (out_dtype == LQ_BF16) return dispatch<bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-  lq_set_error("linear: unknown out dtype %d", out_dtype);
+                 int ldw, int ldc, int epilogue, hipStream_t stream) {
+  if (epilogue == EPI_NONE) {
+    if (out_dtype == LQ_F32) return dispatch<EPI_NONE, float>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (out_dtype == LQ_BF16) return dispatch<EPI_NONE, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  } else if (epilogue == EPI_SWIGLU) {
+    if (N % 16 != 0) {
+      lq_set_error("linear+swiglu: %d interleaved rows are not a multiple of 16", N);
+      return -1;
+    }
+    if (out_dtype == LQ_F32) return dispatch<EPI_SWIGLU, float>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (out_dtype == LQ_BF16) return dispatch<EPI_SWIGLU, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  }
+  lq_set_error("linear: unknown out dtype %d or epilogue %d", out_dtype, epilogue);
   return -1;
 }

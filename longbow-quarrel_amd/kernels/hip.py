@@ -169,6 +169,36 @@ class HipKernels:
                                        c_int(self._rows2d(w, "w")), c_int(self._rows2d(out, "out")),
                                        c_int(1 if self.force_generic else 0), self.stream))
 
+    def linear_swiglu_supported(self, dtype: torch.dtype, rows_out: int, k: int) -> bool:
+        """Whether `linear_swiglu` takes weights of this dtype with `rows_out` (= 2 I) rows and width k."""
+        if self.force_generic or dtype not in _DTYPE_CODE:
+            return False
+        return bool(self.lib.lq_linear_swiglu_supported(c_int(_DTYPE_CODE[dtype]), c_int(rows_out), c_int(k)))
+
+    def linear_swiglu(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+        """out[M, I] = silu(gate) * up with [gate | up] = x . w^T, in one kernel.  w [2 I, K] holds the
+        gate and up rows interleaved in groups of 8: rows 16j..16j+7 gate 8j..8j+7, rows 16j+8..16j+15
+        up 8j..8j+7 (see `interleave_gate_up`)."""
+        self._dev(x, w, out)
+        if x.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+            raise KernelLibraryError("linear_swiglu: 2-D tensors are needed")
+        m, k = x.shape
+        n = w.shape[0]
+        if w.shape[1] != k or tuple(out.shape) != (m, n // 2) or n % 16 != 0 or x.dtype != w.dtype:
+            raise KernelLibraryError(
+                f"linear_swiglu: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.lq_linear_swiglu(_ptr(x), _ptr(w), _ptr(out), c_int(_code(x)), c_int(_code(out)),
+                                              c_int(m), c_int(n), c_int(k), c_int(self._rows2d(x, "x")),
+                                              c_int(self._rows2d(w, "w")), c_int(self._rows2d(out, "out")),
+                                              self.stream))
+
+    @staticmethod
+    def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+        """The weight layout `linear_swiglu` reads (done once, when weights are bound)."""
+        inner, width = gate.shape
+        return torch.stack([gate.view(inner // 8, 8, width), up.view(inner // 8, 8, width)], dim=1) \
+            .reshape(2 * inner, width).contiguous()
+
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
         """out[r, i] = silu(gate_up[r, i]) * gate_up[r, I + i]"""
         self._dev(gate_up, out)

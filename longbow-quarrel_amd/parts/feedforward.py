@@ -20,6 +20,7 @@ class SwiGLU(FeedForward):
         n = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
         n.update(names or {})
         self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
+        self.fused = False
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
@@ -35,16 +36,26 @@ class SwiGLU(FeedForward):
         gate, up = tensors[self.names["gate"]], tensors[self.names["up"]]
         if gate.dtype != up.dtype:
             raise ValueError(f"{self.names['gate']}: gate and up projections are stored in different dtypes")
-        self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
+        kn = env.kernels
+        self.fused = gate.dtype == env.dtype and self.inner % 8 == 0 and \
+            getattr(kn, "linear_swiglu_supported", lambda *a: False)(gate.dtype, 2 * self.inner, self.width)
+        if self.fused:
+            # gate and up rows interleaved so that the product's epilogue can apply silu(g) * u itself
+            self.w_gate_up = kn.interleave_gate_up(gate, up)
+        else:
+            self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = tensors[self.names["down"]].contiguous()
 
     def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         kn = ctx.kernels
         rows = h.shape[0]
-        gu = ctx.ws.alloc((rows, 2 * self.inner), torch.float32)
-        project(kn, ctx, h, self.w_gate_up, gu)
         act = ctx.ws.alloc((rows, self.inner), ctx.dtype)
-        kn.swiglu(gu, act)
+        if self.fused:
+            kn.linear_swiglu(h, self.w_gate_up, act)
+        else:
+            gu = ctx.ws.alloc((rows, 2 * self.inner), torch.float32)
+            project(kn, ctx, h, self.w_gate_up, gu)
+            kn.swiglu(gu, act)
         out = ctx.ws.alloc((rows, self.width), torch.float32)
         project(kn, ctx, act, self.w_down, out)
         return out

@@ -108,7 +108,8 @@ def test_linear_float32(kn, m, n, k):
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("m,n,k", [
     (1, 4096, 4096), (8, 6144, 4096), (16, 1000, 14336), (3, 40, 72), (13, 17, 8),       # skinny
-    (17, 256, 128), (64, 130, 264), (100, 300, 1000), (128, 128, 64), (257, 515, 4096),  # tiled
+    (17, 256, 128), (32, 4096, 4096), (33, 515, 1000), (64, 130, 264), (64, 4096, 14336),  # skinny, more row tiles
+    (65, 256, 128), (100, 300, 1000), (128, 128, 64), (257, 515, 4096),                   # tiled
     (2048, 1024, 512),
 ])
 def test_linear_bfloat16_matrix_cores(kn, out_dtype, m, n, k):
@@ -304,3 +305,23 @@ def test_rope_store_rotates_and_writes_the_right_rows(kn, dtype):
     kn.rope_store(x, None, None, 32, 0, 128, f.to(DEV), i32([5]))
     assert float((x.double().cpu().view(1, 32, 128) - plain.rope(x0.cpu().view(1, 32, 128), [5], f)).abs().max()) \
         < (1e-4 if dtype == torch.float32 else 0.2)
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 33, 64, 65, 300])
+@pytest.mark.parametrize("inner,k", [(16, 8), (328, 96), (1000, 264), (14336, 4096)])
+def test_linear_with_fused_swiglu(kn, m, inner, k):
+    """One kernel for silu(x Wg^T) * (x Wu^T), with gate and up rows interleaved in groups of 8."""
+    if inner == 14336 and m > 64:
+        m = 130
+    x = rnd((m, k), 41, torch.bfloat16)
+    gate, up = rnd((inner, k), 42, torch.bfloat16, 0.05), rnd((inner, k), 43, torch.bfloat16, 0.05)
+    assert kn.linear_swiglu_supported(torch.bfloat16, 2 * inner, k)
+    w = kn.interleave_gate_up(gate, up)
+    out = torch.empty((m, inner), dtype=torch.bfloat16, device=DEV)
+    kn.linear_swiglu(x, w, out)
+    xd = x.double().cpu()
+    want = plain.swiglu(xd @ gate.double().cpu().t(), xd @ up.double().cpu().t())
+    assert rel_err(out, want) < 5e-3
+    out32 = torch.empty((m, inner), dtype=torch.float32, device=DEV)
+    kn.linear_swiglu(x, w, out32)
+    assert rel_err(out32, want) < 2e-5
