@@ -5,10 +5,11 @@ order in which layers run, the final norm and the output head.  `DecoderModel`
 builds the parts through their registries, declares every tensor they bind,
 and runs a step's rows through the schedule.
 
-The schedule is a list of `Run(layer, cache_of)`: the same layer may appear
-more than once (it then runs again with the same weights, writing the same
-cache), and `cache_of = j` lets a layer read the keys and values layer j wrote
-instead of writing its own.
+The schedule is a list of `Run(layer, cache_of)`.  The same layer may appear
+more than once: it then runs again with the same weights, and every run has a
+cache of its own (its inputs differ, so its keys and values do).  `cache_of = j`
+lets a run read what run number j of the schedule (an earlier one) wrote instead
+of writing its own.
 """
 from __future__ import annotations
 
@@ -24,7 +25,7 @@ from .parts.base import (BLOCKS, MATRIX, NORMS, Block, BuildEnv, LayerCache, Nor
 @dataclass(frozen=True)
 class Run:
     layer: int
-    cache_of: Optional[int] = None  # read (never write) the cache of this other layer
+    cache_of: Optional[int] = None  # read (never write) the cache of this earlier run of the schedule
 
 
 @dataclass(frozen=True)
@@ -46,12 +47,13 @@ class DecoderModel:
         self.spec = spec
         self.blocks: List[Block] = [build_part(BLOCKS, b) for b in spec.layers]
         self.final_norm: Norm = build_part(NORMS, spec.final_norm)
-        for run in spec.schedule:
+        for i, run in enumerate(spec.schedule):
             if not 0 <= run.layer < len(self.blocks):
                 raise ValueError(f"schedule names layer {run.layer}, the model has {len(self.blocks)}")
-            if run.cache_of is not None and not 0 <= run.cache_of < len(self.blocks):
-                raise ValueError(f"schedule lets layer {run.layer} read the cache of layer {run.cache_of}, "
-                                 f"the model has {len(self.blocks)}")
+            if run.cache_of is not None:
+                if not 0 <= run.cache_of < i or spec.schedule[run.cache_of].cache_of is not None:
+                    raise ValueError(f"run {i} of the schedule reads the cache of run {run.cache_of}, which is "
+                                     "not an earlier run with a cache of its own")
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
         self.env: Optional[BuildEnv] = None
@@ -82,13 +84,13 @@ class DecoderModel:
 
     # ---- what the cache has to hold -----------------------------------------------
     def cache_needs(self) -> Dict[int, object]:
-        """Layer index -> KVNeed / StateNeed, for the layers that own a cache."""
-        owners = {run.layer if run.cache_of is None else run.cache_of for run in self.spec.schedule}
+        """Run number -> KVNeed / StateNeed, for the runs of the schedule that own a cache."""
         needs = {}
-        for layer in sorted(owners):
-            need = self.blocks[layer].mixer.cache_need()
-            if need is not None:
-                needs[layer] = need
+        for i, run in enumerate(self.spec.schedule):
+            if run.cache_of is None:
+                need = self.blocks[run.layer].mixer.cache_need()
+                if need is not None:
+                    needs[i] = need
         return needs
 
     # ---- one step -------------------------------------------------------------------
@@ -101,9 +103,8 @@ class DecoderModel:
         x = ctx.ws.alloc((ctx.rows, s.width), torch.float32)
         kn.embed(self.embedding, ctx.tokens, x)
         pending: Optional[torch.Tensor] = None
-        for run in s.schedule:
-            owner = run.layer if run.cache_of is None else run.cache_of
-            cache = caches.get(owner)
+        for i, run in enumerate(s.schedule):
+            cache = caches.get(i if run.cache_of is None else run.cache_of)
             if cache is not None and run.cache_of is not None:
                 cache = LayerCache(write=False, k=cache.k, v=cache.v, block_table=cache.block_table,
                                    block_size=cache.block_size, state=cache.state)

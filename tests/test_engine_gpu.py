@@ -1,0 +1,235 @@
+"""The engine on the GPU against the plain implementation, in float32 and in bfloat16: each
+request alone and whole; with the last 32 tokens one by one; in batches of unequal lengths whose
+shorter requests end earlier, one batch after another so that slots are used again; long decoding;
+the first tokens of a sequence; greedy generation through the entry point; toy parts."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import longbow_quarrel_amd as lq
+import plain
+import toy_parts
+from helpers import TINY_A, TINY_B, TINY_C, TOL_BF16, TOL_F32, random_tokens, read_folder, rel_err, write_folder
+from longbow_quarrel_amd.engine import StepEntry
+from longbow_quarrel_amd.loading import random_engine
+from longbow_quarrel_amd.weights import random_tensors
+
+pytestmark = pytest.mark.gpu
+
+# (configuration, std of the random weights): the third has weights large enough that attention is
+# peaked, so that a key read from the wrong place changes the logits by far more than any tolerance
+CASES = {"a": (TINY_A, 0.02), "b": (TINY_B, 0.02), "c_sharp": (TINY_C, 0.15)}
+LENGTHS = (70, 5, 33, 1, 65, 130)
+_cache = {}
+
+
+def setup_case(tmp_path_factory, name, dtype):
+    key = (name, dtype)
+    if key not in _cache:
+        cfg, std = CASES[name]
+        folder = write_folder(tmp_path_factory.mktemp(f"{name}_{dtype}"), cfg, seed=7, std=std)
+        eng = lq.load_engine(folder, dtype=dtype, max_tokens=2048)
+        c, tensors = read_folder(folder)
+        ref = plain.PlainLlama(c, tensors)
+        act = plain.identity if dtype == "float32" else plain.round_bf16
+        reqs = [random_tokens(n, cfg["vocab_size"], 100 + n) for n in LENGTHS]
+        want = [ref.forward(r, act) for r in reqs]
+        _cache[key] = (eng, ref, act, reqs, want, folder)
+    return _cache[key]
+
+
+def tol(dtype):
+    return TOL_F32 if dtype == "float32" else TOL_BF16
+
+
+PARAMS = [(n, d) for n in CASES for d in ("float32", "bfloat16")]
+
+
+@pytest.mark.parametrize("name,dtype", PARAMS)
+def test_each_request_alone_and_whole(tmp_path_factory, name, dtype):
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, name, dtype)
+    for r, w in zip(reqs, want):
+        s = eng.new_sequence()
+        got = eng.step([StepEntry(s, r, range(len(r)))])
+        eng.release(s)
+        assert got.shape == w.shape and rel_err(got, w) < tol(dtype)
+
+
+@pytest.mark.parametrize("name,dtype", PARAMS)
+def test_last_32_tokens_one_by_one(tmp_path_factory, name, dtype):
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, name, dtype)
+    for r, w in zip(reqs, want):
+        if len(r) <= 32:
+            continue
+        s = eng.new_sequence()
+        head = len(r) - 32
+        got = [eng.step([StepEntry(s, r[:head], range(head))])]
+        got += [eng.step([StepEntry(s, [t], [0])]) for t in r[head:]]
+        eng.release(s)
+        got = torch.cat(got)
+        assert rel_err(got, w) < tol(dtype)
+        # the first decoded token and a prompt's end are where a cache fault would show first
+        assert rel_err(got[head - 1], w[head - 1]) < tol(dtype) and rel_err(got[head], w[head]) < tol(dtype)
+
+
+@pytest.mark.parametrize("name,dtype", PARAMS)
+def test_unequal_batches_one_after_another_reuse_slots(tmp_path_factory, name, dtype):
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, name, dtype)
+    used = []
+    for group in ([0, 1, 2], [3, 4, 5], [5, 0]):
+        slots = {i: eng.new_sequence() for i in group}
+        used.append(sorted(slots.values()))
+        split = {i: max(1, len(reqs[i]) - 4 - 3 * j) for j, i in enumerate(group)}
+        out = eng.step([StepEntry(slots[i], reqs[i][: split[i]], range(split[i])) for i in group])
+        at = 0
+        for i in group:
+            assert rel_err(out[at : at + split[i]], want[i][: split[i]]) < tol(dtype)
+            at += split[i]
+        pos = dict(split)
+        for i in group:
+            if pos[i] == len(reqs[i]):
+                eng.release(slots[i])
+        while any(pos[i] < len(reqs[i]) for i in group):
+            live = [i for i in group if pos[i] < len(reqs[i])]
+            out = eng.step([StepEntry(slots[i], [reqs[i][pos[i]]], [0]) for i in live])
+            for j, i in enumerate(live):
+                assert rel_err(out[j], want[i][pos[i]]) < tol(dtype), (i, pos[i])
+                pos[i] += 1
+                if pos[i] == len(reqs[i]):
+                    eng.release(slots[i])
+    assert used[0] == used[1]  # the second batch ran on the slots the first gave back
+    assert eng.cache.slots.taken_count == 0 and all(g.blocks.taken_count == 0 for g in eng.cache.kv_groups)
+
+
+@pytest.mark.parametrize("name,dtype", [("a", "float32"), ("c_sharp", "float32"), ("c_sharp", "bfloat16"), ("b", "bfloat16")])
+def test_long_decoding(tmp_path_factory, name, dtype):
+    """10 prompt tokens, then 290 tokens one by one: across four cache blocks and three attention splits."""
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, name, dtype)
+    cfg = CASES[name][0]
+    toks = random_tokens(300, cfg["vocab_size"], 77)
+    w = ref.forward(toks, act)
+    s = eng.new_sequence()
+    got = [eng.step([StepEntry(s, toks[:10], range(10))])]
+    got += [eng.step([StepEntry(s, [t], [0])]) for t in toks[10:]]
+    eng.release(s)
+    got = torch.cat(got)
+    for lo in range(0, 300, 50):  # localise a fault to the place where it starts
+        assert rel_err(got[lo : lo + 50], w[lo : lo + 50]) < tol(dtype), lo
+
+
+@pytest.mark.parametrize("name,dtype", PARAMS)
+def test_first_tokens_of_a_sequence(tmp_path_factory, name, dtype):
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, name, dtype)
+    toks = reqs[0][:3]
+    w = ref.forward(toks, act)
+    slots = [eng.new_sequence() for _ in range(3)]
+    # three sequences of 1, 2 and 3 tokens in one step, then the shorter ones catch up one token at a time
+    out = eng.step([StepEntry(slots[0], toks[:1], [0]), StepEntry(slots[1], toks[:2], [0, 1]),
+                    StepEntry(slots[2], toks[:3], [0, 1, 2])])
+    for row, p in enumerate([0, 0, 1, 0, 1, 2]):
+        assert rel_err(out[row], w[p]) < tol(dtype)
+    out = eng.step([StepEntry(slots[0], [toks[1]], [0]), StepEntry(slots[1], [toks[2]], [0])])
+    assert rel_err(out[0], w[1]) < tol(dtype) and rel_err(out[1], w[2]) < tol(dtype)
+    for s in slots:
+        eng.release(s)
+
+
+def test_float32_logits_do_not_depend_on_the_cutting_at_all(tmp_path_factory):
+    """In the float32 path every sum has an order fixed by the position alone: bit-equal results."""
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, "c_sharp", "float32")
+    r = reqs[5]
+    s = eng.new_sequence()
+    whole = eng.step([StepEntry(s, r, range(len(r)))])
+    eng.release(s)
+    s, other = eng.new_sequence(), eng.new_sequence()
+    parts = [eng.step([StepEntry(other, reqs[0], []), StepEntry(s, r[:50], range(50))])]
+    parts.append(eng.step([StepEntry(s, r[50:51], [0]), StepEntry(other, [1], [])])[:1])
+    parts.append(eng.step([StepEntry(s, r[51:], range(len(r) - 51))]))
+    eng.release(s)
+    eng.release(other)
+    assert torch.equal(torch.cat(parts), whole)
+
+
+@pytest.mark.parametrize("name,dtype", [("a", "float32"), ("c_sharp", "float32")])
+def test_greedy_generation_through_the_entry_point(tmp_path_factory, name, dtype):
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, name, dtype)
+    prompts = [reqs[1], reqs[3], reqs[2], reqs[0][:9]]
+    expect = []
+    for p in prompts:
+        seq, out = list(p), []
+        for _ in range(10):
+            t = plain.arg_max(ref.forward(seq)[-1])
+            out.append(t)
+            seq.append(t)
+        expect.append(out)
+    for graphs in (False, True):
+        res = lq.generate(eng, prompts, 10, lq.SamplingParams(temperature=0.0), stop_ids=[], max_batch=3,
+                          use_graphs=graphs)
+        assert res.tokens == expect and res.batches == 2
+    # a stop id ends its sequence early and is not returned; the others go on
+    stop = expect[0][4]
+    res = lq.generate(eng, prompts, 10, stop_ids=[stop], max_batch=4)
+    for got, exp in zip(res.tokens, expect):
+        cut = exp.index(stop) if stop in exp else len(exp)
+        assert got == exp[:cut]
+    assert eng.cache.slots.taken_count == 0
+
+
+def test_generation_in_bfloat16_graphs_and_direct_steps_agree(tmp_path_factory):
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, "c_sharp", "bfloat16")
+    prompts = [reqs[1], reqs[2], reqs[4]]
+    for params in (lq.SamplingParams(), lq.SamplingParams(temperature=0.8, top_k=40, top_p=0.95,
+                                                          repetition_penalty=1.1, seed=3)):
+        a = lq.generate(eng, prompts, 70, params, stop_ids=[], use_graphs=False)
+        b = lq.generate(eng, prompts, 70, params, stop_ids=[], use_graphs=True)
+        assert a.tokens == b.tokens and all(len(t) == 70 for t in a.tokens)
+    # a sequence's sampled tokens do not depend on what else is in its batch
+    alone = lq.generate(eng, prompts[:1], 20, lq.SamplingParams(temperature=0.8, seed=3), stop_ids=[])
+    batch = lq.generate(eng, prompts, 20, lq.SamplingParams(temperature=0.8, seed=3), stop_ids=[])
+    assert alone.tokens[0] == batch.tokens[0]
+
+
+def test_command_line_generates_the_same_greedy_tokens(tmp_path_factory):
+    eng, ref, act, reqs, want, folder = setup_case(tmp_path_factory, "a", "float32")
+    prompt = reqs[1]
+    expect = lq.generate(eng, [prompt], 6, stop_ids=[]).tokens[0]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    # eos is id 2 in this configuration; the command line stops there as generation does
+    cut = expect.index(2) if 2 in expect else len(expect)
+    out = subprocess.run([sys.executable, os.path.join(root, "bin", "quarrel"), "-model", folder, "-prompt",
+                          " ".join(map(str, prompt)), "-n", "6", "-temp", "0", "-penalty", "1", "-dtype", "float32"],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert out.stdout.strip().splitlines()[-1].split() == [str(t) for t in expect[:cut]]
+    assert f"{cut} tokens in" in out.stdout
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_parts_on_the_gpu(dtype):
+    """A mixer with state of its own, a feed-forward with routing, another position encoding, a layer
+    that runs twice and one that reads another's cache: registered, built and stepped here."""
+    toy_parts.register_toys()
+    try:
+        cfg = toy_parts.ToyConfig.from_dict(toy_parts.TOY)
+        eng = random_engine(cfg, seed=3, dtype=dtype, max_tokens=512, std=0.2)
+        tensors = {k: v.cpu() for k, v in random_tensors(eng.model.tensor_specs(), 3, eng.dtype, 0.2, device=eng.device).items()}
+        a, b = random_tokens(40, 53, 1), random_tokens(9, 53, 2)
+        wa, wb = (toy_parts.plain_toy(toy_parts.TOY, tensors, t) for t in (a, b))
+        limit = TOL_F32 if dtype == "float32" else 6e-2  # no rounding hooks in the toy's plain twin
+        sa, sb = eng.new_sequence(), eng.new_sequence()
+        out = eng.step([StepEntry(sa, a[:17], range(17)), StepEntry(sb, b[:8], range(8))])
+        assert rel_err(out[:17], wa[:17]) < limit and rel_err(out[17:], wb[:8]) < limit
+        out = eng.step([StepEntry(sa, a[17:18], [0]), StepEntry(sb, b[8:], [0])])
+        assert rel_err(out[0], wa[17]) < limit and rel_err(out[1], wb[8]) < limit
+        eng.release(sb)
+        assert rel_err(eng.step([StepEntry(sa, a[18:], range(22))]), wa[18:]) < limit
+        eng.release(sa)
+        s = eng.new_sequence()
+        assert rel_err(eng.step([StepEntry(s, b, range(9))]), wb) < limit
+        res = lq.generate(eng, [a[:5], b[:3]], 4, stop_ids=[])  # generation falls back to direct steps
+        assert [len(t) for t in res.tokens] == [4, 4]
+    finally:
+        toy_parts.unregister_toys()
