@@ -64,6 +64,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the prefill and the batch 1 / 64 points")
+    ap.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -80,7 +81,7 @@ def main() -> int:
         cfg["num_hidden_layers"] = args.layers
     config = lq.LlamaConfig.from_dict(cfg)
     slot_len = cfg["max_position_embeddings"]
-    max_batch = 64 if not args.no_points else args.batch
+    max_batch = 64 if not (args.no_points or args.prefill_only) else args.batch
     t0 = time.time()
     engine = lq.random_engine(config, seed=0, dtype="bfloat16", max_tokens=max_batch * slot_len, max_slots=max_batch)
     torch.cuda.synchronize()
@@ -114,6 +115,14 @@ def main() -> int:
         backend.close()
         return batch * steps / dt, dt / steps * 1e3, ctx_mean
 
+    if args.prefill_only:
+        slot = engine.new_sequence()
+        engine.step([StepEntry(slot, random_prompt(2048), [2047])])
+        engine.release(slot)
+        slot = engine.new_sequence()
+        engine.step([StepEntry(slot, random_prompt(2048), [2047])])
+        torch.cuda.synchronize()
+        return 0
     value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
     step_bytes = weight_bytes_per_step(config) + args.batch * ctx_mean * kv_bytes_per_token(config)
     achieved = step_bytes / (ms_step * 1e-3) / 1e9

@@ -17,10 +17,15 @@
 // bfloat16 only as MFMA operands (their sum is taken before rounding).
 //
 // Two launch shapes share the inner loop:
-//  * rows:  16 consecutive rows of one sequence for one query head (prompts).
-//  * heads: one row of one sequence for the query heads of one kv head (decoding); keys are
-//    cut into splits of SPLIT positions, aligned to absolute positions, each split a block of its
-//    own, partial results merged by a second kernel in ascending split order.
+//  * rows (prompts): a wave owns QT tiles of 16 consecutive rows of one sequence for one query head
+//    and reuses every key/value fragment it loads for all of them; the waves of a block are the
+//    query heads of one kv head over the same rows, so that they read the same keys at the same time.
+//  * heads (decoding): one row of one sequence, the query heads of one kv head as the 16 columns.
+//    The waves of a block take the chunks of a split of SPLIT positions in turn (wave w: chunks
+//    w, w + NW, ...) and combine their partial results through LDS in wave order.  A sequence longer
+//    than SPLIT has several blocks, merged by a second kernel in ascending split order.  Splits
+//    and chunks are aligned to absolute positions: the order of every sum depends on the row's
+//    position only.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -31,7 +36,7 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr int BS = 64;      // positions per cache block (the only block size this file takes)
-constexpr int SPLIT = 128;  // keys per split when decoding
+constexpr int SPLIT = 1024;  // keys per block when decoding
 
 __device__ inline bf16x8 as_bf16x8(u32x4 v) {
   union {
@@ -42,8 +47,64 @@ __device__ inline bf16x8 as_bf16x8(u32x4 v) {
   return c.b;
 }
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// two floats to packed bfloat16, round to nearest even (v_cvt_pk_bf16_f32)
 __device__ inline unsigned pack_bf16(float lo, float hi) {
-  return (unsigned)f32_to_bf16(lo).bits | ((unsigned)f32_to_bf16(hi).bits << 16);
+  union {
+    bf16x2 b;
+    unsigned u;
+  } c;
+  c.b = __builtin_convertvector((f32x2){lo, hi}, bf16x2);
+  return c.u;
+}
+
+// 2^x for x <= 0 (v_exp_f32; results below the normal range flush to zero, which is what a
+// probability that small is worth)
+__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// One chunk of 32 keys for one query tile: from the raw score tiles s[2] (S^T, lane holds keys
+// (lane/16)*4 + e of each 16-key tile for column lane%16) to the packed probabilities, updating the
+// running maximum m (log2 domain, scores scaled by c = scale * log2 e) and normaliser share l.
+// Returns the factor the output accumulator has to be multiplied with (1 if the maximum stayed).
+// `masked` is wave-uniform: false when every key of the chunk is visible to every column.
+__device__ inline float softmax_chunk(const f32x4 (&s)[2], float c, bool masked, bool col_valid, int t0, int lo,
+                                      int pos, float& m, float& l, u32x4& pw) {
+  const int g = (threadIdx.x & 63) >> 4;
+  float sv[8];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sv[j * 4 + e] = s[j][e];
+  if (masked) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int t = t0 + 16 * j + g * 4 + e;
+        if (!(col_valid && t >= lo && t <= pos)) sv[j * 4 + e] = -INFINITY;
+      }
+  }
+  float cmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+  cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+  cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+  const float m_new = fmaxf(m, cmax * c);  // c > 0: scaling commutes with the maximum
+  const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a column with no key yet
+  const float alpha = fast_exp2(m - m_safe);
+  float psum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    sv[i] = fast_exp2(fmaf(sv[i], c, -m_safe));  // -inf stays -inf, 2^-inf = 0
+    psum += sv[i];
+  }
+  l = l * alpha + psum;
+  m = m_new;
+  pw[0] = pack_bf16(sv[0], sv[1]);
+  pw[1] = pack_bf16(sv[2], sv[3]);
+  pw[2] = pack_bf16(sv[4], sv[5]);
+  pw[3] = pack_bf16(sv[6], sv[7]);
+  return alpha;
 }
 
 struct AttnArgs {
@@ -68,10 +129,6 @@ struct AttnArgs {
   int nsplit;
 };
 
-// The shared inner loop.  Query column c = lane % 16 is valid if c < ncols; its position is
-// p_c, its first key lo_c.  Keys t_begin..t_end (inclusive) are walked; t_begin is a multiple of 32.
-// On return o[dt][e] holds the unnormalised O^T[dt*16 + (lane/16)*4 + e][c], m the running maximum
-// (in the log2 domain) and l this lane's share of the normaliser (to be summed over lane/16).
 // One chunk's operands as they come from memory: 16 bytes a lane for each K fragment, two 8-byte
 // pieces a lane for each V^T fragment.
 template <int HD>
@@ -98,192 +155,389 @@ __device__ inline void load_chunk(const AttnArgs& a, int kvh, long long blk, int
   }
 }
 
-template <int HD>
-__device__ inline void attend(const AttnArgs& a, const bf16x8 (&qf)[HD / 32], int kvh, const int* table,
-                              int t_begin, int t_end, bool col_valid, int p_c, int lo_c,
-                              f32x4 (&o)[HD / 16], float& m, float& l) {
+// What a wave carries for each of its QT query tiles.  Column c = lane % 16 of tile qt is valid if
+// valid[qt]; its position is pos[qt], its first key lo[qt].  o[qt][dt][e] is the unnormalised
+// O^T[dt*16 + (lane/16)*4 + e][c], m the running maximum (log2 domain), l this lane's share of
+// the normaliser (to be summed over lane/16).
+template <int HD, int QT>
+struct QTiles {
+  bf16x8 q[QT][HD / 32];
+  f32x4 o[QT][HD / 16];
+  float m[QT], l[QT];
+  bool valid[QT];
+  int pos[QT], lo[QT];
+  int last_key[QT];   // largest position any column of the tile may see (wave-uniform)
+  int first_key[QT];  // smallest (wave-uniform)
+  int free_to[QT];    // chunks that end at or before this key and start at or after free_from are
+  int free_from[QT];  //   visible to every column: no masking needed (wave-uniform; free_to = -1: never)
+};
+
+// Walks chunks t_first, t_first + t_step, ... while <= t_end (all multiples of 32).  Keys beyond
+// t_written were never written and are kept out of the second product.
+template <int HD, int QT>
+__device__ inline void attend(const AttnArgs& a, QTiles<HD, QT>& w, int kvh, const int* table, int t_first,
+                              int t_step, int t_end, int t_written) {
   const int lane = threadIdx.x & 63, g = lane >> 4;
+  if (t_first > t_end) return;
   // the next chunk's keys and values are already on their way while this chunk is computed, and
   // the block number of the chunk after that while those are loaded
   ChunkRegs<HD> cur, nxt;
-  long long blk_next = table[t_begin / BS];
-  load_chunk<HD>(a, kvh, blk_next, t_begin % BS, nxt);
-  blk_next = (t_begin + 32 <= t_end) ? table[(t_begin + 32) / BS] : 0;
-  for (int t0 = t_begin; t0 <= t_end; t0 += 32) {
+  long long blk_next = table[t_first / BS];
+  load_chunk<HD>(a, kvh, blk_next, t_first % BS, nxt);
+  blk_next = (t_first + t_step <= t_end) ? table[(t_first + t_step) / BS] : 0;
+  for (int t0 = t_first; t0 <= t_end; t0 += t_step) {
     cur = nxt;
-    if (t0 + 32 <= t_end) {
-      load_chunk<HD>(a, kvh, blk_next, (t0 + 32) % BS, nxt);
-      blk_next = (t0 + 64 <= t_end) ? table[(t0 + 64) / BS] : 0;
+    if (t0 + t_step <= t_end) {
+      load_chunk<HD>(a, kvh, blk_next, (t0 + t_step) % BS, nxt);
+      blk_next = (t0 + 2 * t_step <= t_end) ? table[(t0 + 2 * t_step) / BS] : 0;
     }
-    f32x4 s[2];
+    // values of keys that were never written must not reach the product (0 * garbage may be NaN)
+    if (t0 + 31 > t_written) {
+      const int ta = t0 + g * 4, tb = t0 + 16 + g * 4;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      s[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < HD / 32; ++kk)
-        s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.k[j][kk]), qf[kk], s[j], 0, 0, 0);
-    }
-    float sv[8];
-    float cmax = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int t = t0 + 16 * j + g * 4 + e;
-        const bool ok = col_valid && t >= lo_c && t <= p_c;
-        const float v = ok ? s[j][e] * a.scale_log2 : -INFINITY;
-        sv[j * 4 + e] = v;
-        cmax = fmaxf(cmax, v);
+      for (int dt = 0; dt < HD / 16; ++dt) {
+        if (ta + 0 > t_written) cur.v[dt][0][0] &= 0xffff0000u;
+        if (ta + 1 > t_written) cur.v[dt][0][0] &= 0x0000ffffu;
+        if (ta + 2 > t_written) cur.v[dt][0][1] &= 0xffff0000u;
+        if (ta + 3 > t_written) cur.v[dt][0][1] &= 0x0000ffffu;
+        if (tb + 0 > t_written) cur.v[dt][1][0] &= 0xffff0000u;
+        if (tb + 1 > t_written) cur.v[dt][1][0] &= 0x0000ffffu;
+        if (tb + 2 > t_written) cur.v[dt][1][1] &= 0xffff0000u;
+        if (tb + 3 > t_written) cur.v[dt][1][1] &= 0x0000ffffu;
       }
-    cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
-    cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
-    const float m_new = fmaxf(m, cmax);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a column with no key yet
-    const float alpha = exp2f(m - m_safe);
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      sv[i] = exp2f(sv[i] - m_safe);
-      psum += sv[i];
     }
-    l = l * alpha + psum;
-    m = m_new;
-    u32x4 pw;
-    pw[0] = pack_bf16(sv[0], sv[1]);
-    pw[1] = pack_bf16(sv[2], sv[3]);
-    pw[2] = pack_bf16(sv[4], sv[5]);
-    pw[3] = pack_bf16(sv[6], sv[7]);
-    const bf16x8 pb = as_bf16x8(pw);
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      if (t0 > w.last_key[qt] || t0 + 31 < w.first_key[qt]) continue;  // nothing of this chunk is visible
+      f32x4 s[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        s[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < HD / 32; ++kk)
+          s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.k[j][kk]), w.q[qt][kk], s[j], 0, 0, 0);
+      }
+      const bool masked = !(t0 + 31 <= w.free_to[qt] && t0 >= w.free_from[qt]);
+      u32x4 pw;
+      const float alpha = softmax_chunk(s, a.scale_log2, masked, w.valid[qt], t0, w.lo[qt], w.pos[qt], w.m[qt],
+                                        w.l[qt], pw);
+      const bf16x8 pb = as_bf16x8(pw);
+      if (!__all(alpha == 1.0f)) {  // the maximum moved for some column: rescale what has been summed
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w.o[qt][dt][e] *= alpha;
+      }
+#pragma unroll
+      for (int dt = 0; dt < HD / 16; ++dt) {
+        u32x4 vv;
+        vv[0] = cur.v[dt][0][0];
+        vv[1] = cur.v[dt][0][1];
+        vv[2] = cur.v[dt][1][0];
+        vv[3] = cur.v[dt][1][1];
+        w.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vv), pb, w.o[qt][dt], 0, 0, 0);
+      }
+    }
+  }
+}
 
-    // keys past t_end lie in the block but were never written: their values must not reach the
-    // product (0 * garbage may be NaN), so they are zeroed
-    const bool tail = t0 + 31 > t_end;
+template <int HD, int QT>
+__device__ inline void init_tiles(QTiles<HD, QT>& w) {
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt) {
-      u32x2 v0 = cur.v[dt][0];
-      u32x2 v1 = cur.v[dt][1];
-      if (tail) {
-        const int ta = t0 + g * 4, tb = t0 + 16 + g * 4;
-        if (ta + 0 > t_end) v0[0] &= 0xffff0000u;
-        if (ta + 1 > t_end) v0[0] &= 0x0000ffffu;
-        if (ta + 2 > t_end) v0[1] &= 0xffff0000u;
-        if (ta + 3 > t_end) v0[1] &= 0x0000ffffu;
-        if (tb + 0 > t_end) v1[0] &= 0xffff0000u;
-        if (tb + 1 > t_end) v1[0] &= 0x0000ffffu;
-        if (tb + 2 > t_end) v1[1] &= 0xffff0000u;
-        if (tb + 3 > t_end) v1[1] &= 0x0000ffffu;
-      }
-      u32x4 vv;
-      vv[0] = v0[0];
-      vv[1] = v0[1];
-      vv[2] = v1[0];
-      vv[3] = v1[1];
+  for (int qt = 0; qt < QT; ++qt) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[dt][e] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vv), pb, o[dt], 0, 0, 0);
-    }
+    for (int dt = 0; dt < HD / 16; ++dt) w.o[qt][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    w.m[qt] = -INFINITY;
+    w.l[qt] = 0.f;
   }
 }
 
 // ------------------------------------------------------------------ rows (prompts)
+// Block = NW waves = NW query heads of one kv head over the same QT * 16 rows.  The block walks
+// the keys one cache block (64 positions) at a time: all threads copy the block's K [64][HD] and
+// V^T [HD][64] from memory into padded LDS (next block's copy in registers while the current one is
+// multiplied), and every wave reads its MFMA operands from there, so a key is fetched once for
+// all the heads that share it.  LDS rows are padded (K: +16 bytes, V^T: +16 bytes) so that the
+// operand reads of a quarter wave fall into distinct banks.
 template <int HD>
-__global__ __launch_bounds__(64) void attn_rows_kernel(AttnArgs a) {
-  // find this block's tile: tiles of 16 rows, counted sequence by sequence
+struct RowsLds {
+  static constexpr int K_STRIDE = HD * 2 + 16;   // bytes per key row
+  static constexpr int V_STRIDE = BS * 2 + 16;   // bytes per d row
+  static constexpr int K_BYTES = BS * K_STRIDE;
+  static constexpr int V_BYTES = HD * V_STRIDE;
+  static constexpr int STAGE = K_BYTES + V_BYTES;
+  static constexpr int PIECES = HD * 8;          // 16-byte pieces of K (and of V^T) in one cache block
+};
+
+template <int HD, int QT, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_rows_kernel(AttnArgs a, int heads_per_block_group) {
+  using L = RowsLds<HD>;
+  constexpr int ROWS = QT * 16;
+  constexpr int THREADS = NW * 64;
+  constexpr int PER_THREAD = (L::PIECES + THREADS - 1) / THREADS;  // pieces of K, and of V, per thread
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  // find this block's tile: tiles of ROWS rows, counted sequence by sequence
   int t = blockIdx.x, b = 0, r0 = -1, nrows = 0;
   for (; b < a.batch; ++b) {
     const int begin = a.cu_rows[b], n = a.cu_rows[b + 1] - begin;
-    const int tiles = (n + 15) / 16;
+    const int tiles = (n + ROWS - 1) / ROWS;
     if (t < tiles) {
-      r0 = begin + t * 16;
-      nrows = min(16, n - t * 16);
+      r0 = begin + t * ROWS;
+      nrows = min(ROWS, n - t * ROWS);
       break;
     }
     t -= tiles;
   }
-  if (r0 < 0) return;
-  const int lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
-  const int h = blockIdx.y, kvh = h / (a.nh / a.nkv);
+  if (r0 < 0) return;  // the whole block
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c16 = lane & 15, g = lane >> 4;
+  const int G = a.nh / a.nkv;
+  // blockIdx.y = kv head * groups + group, a group being NW consecutive query heads of the kv head
+  const int kvh = blockIdx.y / heads_per_block_group;
+  const int hq = (blockIdx.y % heads_per_block_group) * NW + wave;
+  const bool wave_active = hq < G;  // an idle wave still copies and meets the barriers
+  const int h = kvh * G + min(hq, G - 1);
   const int* table = a.block_table + (long long)a.seq_slot[b] * a.bt_stride;
   const int p0 = a.row_pos[r0];
-  const bool col_valid = c16 < nrows;
-  const int p_c = p0 + min(c16, nrows - 1);
-  const int lo_c = (a.window > 0 && p_c >= a.window) ? p_c - a.window + 1 : 0;
-  const int lo_tile = (a.window > 0 && p0 >= a.window) ? p0 - a.window + 1 : 0;
 
-  bf16x8 qf[HD / 32];
-  {
-    const bf16_t* qr = a.q + (long long)(r0 + min(c16, nrows - 1)) * a.ldq + h * HD + g * 8;
+  QTiles<HD, QT> w;
+  init_tiles<HD, QT>(w);
 #pragma unroll
-    for (int kk = 0; kk < HD / 32; ++kk) qf[kk] = as_bf16x8(*(const u32x4*)(qr + kk * 32));
+  for (int qt = 0; qt < QT; ++qt) {
+    const int rows_here = min(16, nrows - qt * 16);  // may be <= 0: the tile is empty
+    const int rc = qt * 16 + min(c16, max(rows_here, 1) - 1);
+    const int row = r0 + min(rc, nrows - 1);
+    w.valid[qt] = wave_active && c16 < rows_here;
+    w.pos[qt] = p0 + min(rc, nrows - 1);
+    w.lo[qt] = (a.window > 0 && w.pos[qt] >= a.window) ? w.pos[qt] - a.window + 1 : 0;
+    const int first_pos = p0 + min(qt * 16, nrows - 1);
+    w.last_key[qt] = (wave_active && rows_here > 0) ? p0 + qt * 16 + rows_here - 1 : -1;
+    w.first_key[qt] = (a.window > 0 && first_pos >= a.window) ? first_pos - a.window + 1 : 0;
+    // a full tile of 16 rows: keys up to its first row's position and from its last row's window
+    // start on are visible to all of its columns
+    const int last_pos = p0 + qt * 16 + rows_here - 1;
+    w.free_to[qt] = (wave_active && rows_here == 16) ? first_pos : -1;
+    w.free_from[qt] = (a.window > 0 && last_pos >= a.window) ? last_pos - a.window + 1 : 0;
+    const bf16_t* qr = a.q + (long long)row * a.ldq + h * HD + g * 8;
+#pragma unroll
+    for (int kk = 0; kk < HD / 32; ++kk) w.q[qt][kk] = as_bf16x8(*(const u32x4*)(qr + kk * 32));
   }
-  f32x4 o[HD / 16];
+  const int t_end = p0 + nrows - 1;  // the last key anyone here sees, and the last one written
+  const int lo_tile = (a.window > 0 && p0 >= a.window) ? p0 - a.window + 1 : 0;
+  const int blk_first = lo_tile / BS, blk_last = t_end / BS;
+
+  u32x4 rk[PER_THREAD], rv[PER_THREAD];
+  auto fetch = [&](int lb) {
+    const long long blk = table[lb];
+    const bf16_t* kb = a.kcache + (blk * a.nkv + kvh) * (long long)(BS * HD);
+    const bf16_t* vb = a.vcache + (blk * a.nkv + kvh) * (long long)(HD * BS);
 #pragma unroll
-  for (int dt = 0; dt < HD / 16; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-  attend<HD>(a, qf, kvh, table, (lo_tile / 32) * 32, p0 + nrows - 1, col_valid, p_c, lo_c, o, m, l);
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  if (!col_valid) return;
-  const float inv = 1.0f / l;
-  bf16_t* orow = a.out + (long long)(r0 + c16) * a.ldo + h * HD + g * 4;
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int pc = tid + i * THREADS;
+      if (pc < L::PIECES) {
+        rk[i] = *(const u32x4*)(kb + pc * 8);
+        rv[i] = *(const u32x4*)(vb + pc * 8);
+      }
+    }
+  };
+  auto stash = [&](int lb, unsigned char* stage) {
+    // values of keys that were never written must not reach the product (0 * garbage may be NaN)
+    const int base_key = lb * BS;
+    const bool tail = base_key + BS - 1 > t_end;
 #pragma unroll
-  for (int dt = 0; dt < HD / 16; ++dt) {
-    u32x2 w;
-    w[0] = pack_bf16(o[dt][0] * inv, o[dt][1] * inv);
-    w[1] = pack_bf16(o[dt][2] * inv, o[dt][3] * inv);
-    *(u32x2*)(orow + dt * 16) = w;
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int pc = tid + i * THREADS;
+      if (pc < L::PIECES) {
+        const int key = pc / (HD / 8), part = pc % (HD / 8);
+        *(u32x4*)(stage + key * L::K_STRIDE + part * 16) = rk[i];
+        const int d = pc >> 3, vpart = pc & 7;
+        u32x4 v = rv[i];
+        if (tail) {
+          const int k0 = base_key + vpart * 8;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (k0 + 2 * e > t_end) v[e] &= 0xffff0000u;
+            if (k0 + 2 * e + 1 > t_end) v[e] &= 0x0000ffffu;
+          }
+        }
+        *(u32x4*)(stage + L::K_BYTES + d * L::V_STRIDE + vpart * 16) = v;
+      }
+    }
+  };
+
+  fetch(blk_first);
+  stash(blk_first, smem);
+  __syncthreads();
+  for (int lb = blk_first; lb <= blk_last; ++lb) {
+    unsigned char* cur = smem + ((lb - blk_first) & 1) * L::STAGE;
+    unsigned char* nxt = smem + ((lb - blk_first + 1) & 1) * L::STAGE;
+    const bool more = lb < blk_last;
+    if (more) fetch(lb + 1);  // in flight while this block is multiplied
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int t0 = lb * BS + half * 32;
+      if (t0 > t_end) break;
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        if (t0 > w.last_key[qt] || t0 + 31 < w.first_key[qt]) continue;  // nothing of this chunk is visible
+        f32x4 sc[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          sc[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          const unsigned char* kr = cur + (half * 32 + 16 * j + c16) * L::K_STRIDE + g * 16;
+#pragma unroll
+          for (int kk = 0; kk < HD / 32; ++kk)
+            sc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(*(const u32x4*)(kr + kk * 64)), w.q[qt][kk],
+                                                            sc[j], 0, 0, 0);
+        }
+        const bool masked = !(t0 + 31 <= w.free_to[qt] && t0 >= w.free_from[qt]);
+        u32x4 pw;
+        const float alpha = softmax_chunk(sc, a.scale_log2, masked, w.valid[qt], t0, w.lo[qt], w.pos[qt], w.m[qt],
+                                          w.l[qt], pw);
+        const bf16x8 pb = as_bf16x8(pw);
+        if (!__all(alpha == 1.0f)) {  // the maximum moved for some column: rescale what has been summed
+#pragma unroll
+          for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w.o[qt][dt][e] *= alpha;
+        }
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; ++dt) {
+          const unsigned char* vr = cur + L::K_BYTES + (dt * 16 + c16) * L::V_STRIDE + half * 64 + g * 8;
+          const u32x2 v0 = *(const u32x2*)vr;
+          const u32x2 v1 = *(const u32x2*)(vr + 32);
+          u32x4 vv;
+          vv[0] = v0[0];
+          vv[1] = v0[1];
+          vv[2] = v1[0];
+          vv[3] = v1[1];
+          w.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vv), pb, w.o[qt][dt], 0, 0, 0);
+        }
+      }
+    }
+    if (more) stash(lb + 1, nxt);  // nobody reads nxt: its last readers passed the barrier below one round ago
+    __syncthreads();
+  }
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    float l = w.l[qt];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!w.valid[qt]) continue;
+    const float inv = 1.0f / l;
+    bf16_t* orow = a.out + (long long)(r0 + qt * 16 + c16) * a.ldo + h * HD + g * 4;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+      u32x2 ww;
+      ww[0] = pack_bf16(w.o[qt][dt][0] * inv, w.o[qt][dt][1] * inv);
+      ww[1] = pack_bf16(w.o[qt][dt][2] * inv, w.o[qt][dt][3] * inv);
+      *(u32x2*)(orow + dt * 16) = ww;
+    }
   }
 }
 
+template <int HD, int QT, int NW>
+int launch_rows(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
+  using L = RowsLds<HD>;
+  constexpr int ROWS = QT * 16;
+  const size_t smem = 2 * (size_t)L::STAGE;
+  auto kernel = attn_rows_kernel<HD, QT, NW>;
+  static bool configured = false;
+  if (!configured && smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      lq_set_error("attention: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+      return -2;
+    }
+    configured = true;
+  }
+  dim3 grid(lq_ceil_div(rows, ROWS) + a.batch, a.nkv * groups);
+  kernel<<<grid, NW * 64, smem, stream>>>(a, groups);
+  LQ_CHECK_LAUNCH("attention(mfma rows)");
+  return 0;
+}
+
 // ------------------------------------------------------------------ heads (decoding)
-template <int HD>
-__global__ __launch_bounds__(64) void attn_heads_kernel(AttnArgs a) {
-  const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
-  const int lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
+// Block = NW waves over one split of one (sequence, kv head).  LDS: per wave HD x G floats of
+// partial output (the valid columns only), G maxima, G normalisers.
+template <int HD, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int G = a.nh / a.nkv;
+  float* lds_o = lds;                    // [NW][HD][G]
+  float* lds_m = lds + NW * HD * G;      // [NW][G]
+  float* lds_l = lds_m + NW * G;         // [NW][G]
+  const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, g = lane >> 4;
   const int r = a.cu_rows[b];
   const int p = a.row_pos[r];
   const int lo = (a.window > 0 && p >= a.window) ? p - a.window + 1 : 0;
-  const int t_begin = max(split * SPLIT, (lo / 32) * 32);
-  const int t_end = min(split * SPLIT + SPLIT - 1, p);
-  if (t_begin > t_end || split * SPLIT + SPLIT - 1 < lo) return;
+  const int s_begin = max(split * SPLIT, (lo / 32) * 32);
+  const int s_end = min(split * SPLIT + SPLIT - 1, p);
+  if (s_begin > s_end) return;  // the whole block: this split holds no key of the row
   const int* table = a.block_table + (long long)a.seq_slot[b] * a.bt_stride;
-  const bool col_valid = c16 < G;
   const int h = kvh * G + min(c16, G - 1);
 
-  bf16x8 qf[HD / 32];
+  QTiles<HD, 1> w;
+  init_tiles<HD, 1>(w);
+  w.valid[0] = c16 < G;
+  w.pos[0] = p;
+  w.lo[0] = lo;
+  w.last_key[0] = p;
+  w.first_key[0] = lo;
+  w.free_to[0] = -1;  // columns beyond the group's heads are never valid: always the masked path
+  w.free_from[0] = 0;
   {
     const bf16_t* qr = a.q + (long long)r * a.ldq + h * HD + g * 8;
 #pragma unroll
-    for (int kk = 0; kk < HD / 32; ++kk) qf[kk] = as_bf16x8(*(const u32x4*)(qr + kk * 32));
+    for (int kk = 0; kk < HD / 32; ++kk) w.q[0][kk] = as_bf16x8(*(const u32x4*)(qr + kk * 32));
   }
-  f32x4 o[HD / 16];
-#pragma unroll
-  for (int dt = 0; dt < HD / 16; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-  attend<HD>(a, qf, kvh, table, t_begin, t_end, col_valid, p, lo, o, m, l);
+  // chunk numbering is absolute within the split, so that a wave's chunks depend on positions only
+  int t_first = split * SPLIT + wave * 32;
+  while (t_first < s_begin) t_first += NW * 32;
+  attend<HD, 1>(a, w, kvh, table, t_first, NW * 32, s_end, p);
+  float l = w.l[0];
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
-  if (!col_valid) return;
-  if (a.nsplit == 1) {
-    const float inv = 1.0f / l;
-    bf16_t* orow = a.out + (long long)r * a.ldo + h * HD + g * 4;
+
+  // combine the waves' partial results in wave order
+  if (c16 < G) {
+    float* my_o = lds_o + (long long)wave * HD * G;
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt) {
-      u32x2 w;
-      w[0] = pack_bf16(o[dt][0] * inv, o[dt][1] * inv);
-      w[1] = pack_bf16(o[dt][2] * inv, o[dt][3] * inv);
-      *(u32x2*)(orow + dt * 16) = w;
+    for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) my_o[(dt * 16 + g * 4 + e) * G + c16] = w.o[0][dt][e];
+    if (g == 0) {
+      lds_m[wave * G + c16] = w.m[0];
+      lds_l[wave * G + c16] = l;
     }
-    return;
   }
-  const long long slot = ((long long)r * a.nh + h) * a.nsplit + split;
-  float* po = a.part_o + slot * HD + g * 4;
+  __syncthreads();
+  // every thread finishes some (d, column) pairs: HD * G of them over NW * 64 threads
+  for (int idx = threadIdx.x; idx < HD * G; idx += NW * 64) {
+    const int d = idx / G, c = idx - d * G;
+    float M = -INFINITY;
 #pragma unroll
-  for (int dt = 0; dt < HD / 16; ++dt) *(f32x4*)(po + dt * 16) = o[dt];
-  if (g == 0) {
-    a.part_ml[slot * 2] = m;
-    a.part_ml[slot * 2 + 1] = l;
+    for (int j = 0; j < NW; ++j) M = fmaxf(M, lds_m[j * G + c]);
+    float acc = 0.f, L = 0.f;
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+      const float mj = lds_m[j * G + c];
+      const float wgt = (mj == -INFINITY) ? 0.f : exp2f(mj - M);
+      acc += wgt * lds_o[((long long)j * HD + d) * G + c];
+      L += wgt * lds_l[j * G + c];
+    }
+    const int hh = kvh * G + c;
+    if (a.nsplit == 1) {
+      a.out[(long long)r * a.ldo + hh * HD + d] = f32_to_bf16(acc / L);
+    } else {
+      const long long slot = ((long long)r * a.nh + hh) * a.nsplit + split;
+      a.part_o[slot * HD + d] = acc;
+      if (d == 0) {
+        a.part_ml[slot * 2] = M;
+        a.part_ml[slot * 2 + 1] = L;
+      }
+    }
   }
 }
 
@@ -304,12 +558,12 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(AttnArgs a) {
 #pragma unroll
   for (int j = 0; j < HD / 64 + 1; ++j) acc[j] = 0.f;
   for (int s = s_first; s <= s_last; ++s) {
-    const float w = exp2f(a.part_ml[(base + s) * 2] - M);
-    L += w * a.part_ml[(base + s) * 2 + 1];
+    const float wgt = exp2f(a.part_ml[(base + s) * 2] - M);
+    L += wgt * a.part_ml[(base + s) * 2 + 1];
 #pragma unroll
     for (int j = 0; j < HD / 64 + 1; ++j) {
       const int d = lane + 64 * j;
-      if (d < HD) acc[j] += w * a.part_o[(base + s) * HD + d];
+      if (d < HD) acc[j] += wgt * a.part_o[(base + s) * HD + d];
     }
   }
   const float inv = 1.0f / L;
@@ -322,14 +576,26 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(AttnArgs a) {
 
 template <int HD>
 int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
+  const int G = a.nh / a.nkv;
   if (!decode) {
-    dim3 grid(lq_ceil_div(rows, 16) + a.batch, a.nh);
-    attn_rows_kernel<HD><<<grid, 64, 0, stream>>>(a);
-    LQ_CHECK_LAUNCH("attention(mfma rows)");
-    return 0;
+    constexpr int QT = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
+    if (G >= 4) return launch_rows<HD, QT, 4>(a, rows, lq_ceil_div(G, 4), stream);
+    if (G >= 2) return launch_rows<HD, QT, 2>(a, rows, lq_ceil_div(G, 2), stream);
+    return launch_rows<HD, QT, 1>(a, rows, 1, stream);
   }
+  // as many waves (at most 16) as keep the partial outputs within 48 KiB of LDS
+  const int per_wave = (HD * G + 2 * G) * (int)sizeof(float);
+  const int fit = (48 * 1024) / per_wave;
   dim3 grid(a.batch, a.nkv, a.nsplit);
-  attn_heads_kernel<HD><<<grid, 64, 0, stream>>>(a);
+  if (fit >= 16 && HD <= 64) {
+    attn_heads_kernel<HD, 16><<<grid, 16 * 64, (size_t)16 * per_wave, stream>>>(a);
+  } else if (fit >= 8) {
+    attn_heads_kernel<HD, 8><<<grid, 8 * 64, (size_t)8 * per_wave, stream>>>(a);
+  } else if (fit >= 4) {
+    attn_heads_kernel<HD, 4><<<grid, 4 * 64, (size_t)4 * per_wave, stream>>>(a);
+  } else {
+    attn_heads_kernel<HD, 2><<<grid, 2 * 64, (size_t)2 * per_wave, stream>>>(a);
+  }
   LQ_CHECK_LAUNCH("attention(mfma heads)");
   if (a.nsplit > 1) {
     dim3 mgrid(a.batch, a.nh);

@@ -278,6 +278,123 @@ int launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, in
   return 0;
 }
 
+// ------------------------------------------------------------------ skinny, at most 16 rows
+// One block per compute unit (or a small multiple): the N columns are dealt out in equal runs, so
+// every compute unit streams the same number of weight bytes; a block walks its run in tiles of
+// 16 columns.  The block's KW waves own contiguous K slices and keep their x fragments in
+// registers across the tiles, so x is read once per block and each tile costs weight loads only
+// (all of a tile's loads are in flight together).  Partial tiles meet in LDS, summed in wave order.
+constexpr int V3_KB = 8;    // k-steps (of 32) whose x fragments a wave holds at a time
+constexpr int V3_MAXT = 8;  // tiles a block may own
+
+template <int KW, int EPI, typename TO>
+__global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16_t* __restrict__ X, int ldx,
+                                                                      const bf16_t* __restrict__ W, int ldw,
+                                                                      TO* __restrict__ C, int ldc, int M, int N,
+                                                                      int K, int cols_per_block, int ks_per_wave) {
+  __shared__ float red[2][KW][256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int g = lane >> 4, c16 = lane & 15;
+  const int col_begin = blockIdx.x * cols_per_block;
+  const int col_end = min(N, col_begin + cols_per_block);
+  if (col_begin >= N) return;
+  const int ntiles = (col_end - col_begin + 15) / 16;
+  const int k_wave = wave * ks_per_wave * 32;                 // this wave's slice [k_wave, k_stop)
+  const int k_stop = min(K, k_wave + ks_per_wave * 32);
+  const bf16_t* xp = X + (long long)min(c16, M - 1) * ldx;  // k below already holds the lane's g * 8
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  f32x4 acc[V3_MAXT];
+#pragma unroll
+  for (int t = 0; t < V3_MAXT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  for (int kb = k_wave; kb < k_stop; kb += V3_KB * 32) {
+    u32x4 xv[V3_KB];
+#pragma unroll
+    for (int s = 0; s < V3_KB; ++s) {
+      const int k = kb + s * 32 + g * 8;
+      xv[s] = (k < k_stop) ? *(const u32x4*)(xp + k) : zero;
+    }
+#pragma unroll
+    for (int t = 0; t < V3_MAXT; ++t) {
+      if (t < ntiles) {
+        const int nrow = min(col_begin + t * 16 + c16, col_end - 1);
+        const bf16_t* wp = W + (long long)nrow * ldw;
+        u32x4 wv[V3_KB];
+#pragma unroll
+        for (int s = 0; s < V3_KB; ++s) {
+          const int k = kb + s * 32 + g * 8;
+          wv[s] = (k < k_stop) ? *(const u32x4*)(wp + k) : zero;
+        }
+#pragma unroll
+        for (int s = 0; s < V3_KB; ++s)
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[s]), as_bf16x8(wv[s]), acc[t], 0, 0, 0);
+      }
+    }
+  }
+  // acc[t][e] = C[(lane / 16) * 4 + e][col_begin + 16 t + lane % 16], partial over this wave's k
+#pragma unroll
+  for (int t = 0; t < V3_MAXT; ++t) {
+    if (t < ntiles) {
+      float(*r)[256] = red[t & 1];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[wave][e * 64 + lane] = acc[t][e];
+      __syncthreads();  // also: the buffer written two tiles ago has been read by then
+      if (wave == t % KW) {
+        const int col = col_begin + t * 16 + c16;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float s = 0.f;
+#pragma unroll
+          for (int w = 0; w < KW; ++w) s += r[w][e * 64 + lane];
+          const int row = g * 4 + e;
+          if (EPI == EPI_SWIGLU) {
+            const float up = __shfl(s, lane + 8, 64);
+            if (c16 < 8 && row < M && col + 8 < col_end)
+              store_out<TO>(C + (long long)row * ldc + ((col_begin + t * 16) >> 1) + c16, silu_mul(s, up));
+          } else {
+            if (row < M && col < col_end) store_out<TO>(C + (long long)row * ldc + col, s);
+          }
+        }
+      }
+    }
+  }
+}
+
+static int lq_compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      n = prop.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+
+template <int EPI, typename TO>
+int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc,
+                     hipStream_t stream) {
+  constexpr int KW = 16;
+  const int cus = lq_compute_units();
+  // equal runs of columns, in units of 16 (8 without the paired epilogue), at most V3_MAXT tiles each
+  const int unit = EPI == EPI_SWIGLU ? 16 : 8;
+  int blocks = cus;
+  int cols = lq_ceil_div(lq_ceil_div(N, blocks), unit) * unit;
+  while (cols > V3_MAXT * 16) {
+    blocks += cus;
+    cols = lq_ceil_div(lq_ceil_div(N, blocks), unit) * unit;
+  }
+  const int grid = lq_ceil_div(N, cols);
+  const int ksteps = lq_ceil_div(K, 32);
+  const int ks_per_wave = lq_ceil_div(ksteps, KW);
+  gemm_bf16_skinny_v3_kernel<KW, EPI, TO><<<grid, KW * 64, 0, stream>>>(
+      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, cols, ks_per_wave);
+  LQ_CHECK_LAUNCH("linear(mfma skinny v3)");
+  return 0;
+}
+
 template <int MT, int EPI, typename TO>
 int pick_skinny(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
                 hipStream_t stream) {
@@ -294,7 +411,11 @@ int pick_skinny(const void* x, const void* w, void* out, int M, int N, int K, in
 template <int EPI, typename TO>
 int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
              hipStream_t stream) {
-  if (M <= 16) return pick_skinny<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  if (M <= 16) {
+    // wide enough to give every compute unit a run of columns: the balanced kernel; else the simple one
+    if (N >= 8 * lq_compute_units() && K >= 512) return launch_skinny_v3<EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    return pick_skinny<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  }
   if (M <= 32) return pick_skinny<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   if (M <= 64) return pick_skinny<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   return launch_tiled<2, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);

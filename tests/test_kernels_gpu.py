@@ -108,6 +108,7 @@ def test_linear_float32(kn, m, n, k):
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("m,n,k", [
     (1, 4096, 4096), (8, 6144, 4096), (16, 1000, 14336), (3, 40, 72), (13, 17, 8),       # skinny
+    (5, 2056, 520), (16, 4104, 14336), (8, 128256, 4096), (2, 2048, 8200),                 # skinny, balanced runs
     (17, 256, 128), (32, 4096, 4096), (33, 515, 1000), (64, 130, 264), (64, 4096, 14336),  # skinny, more row tiles
     (65, 256, 128), (100, 300, 1000), (128, 128, 64), (257, 515, 4096),                   # tiled
     (2048, 1024, 512),
