@@ -270,15 +270,16 @@ struct RowsLds {
 };
 
 template <int HD, int QT, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_rows_kernel(AttnArgs a, int heads_per_block_group) {
+__global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_rows_kernel(AttnArgs a, int heads_per_block_group) {
   using L = RowsLds<HD>;
   constexpr int ROWS = QT * 16;
   constexpr int THREADS = NW * 64;
   constexpr int PER_THREAD = (L::PIECES + THREADS - 1) / THREADS;  // pieces of K, and of V, per thread
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-  // find this block's tile: tiles of ROWS rows, counted sequence by sequence
-  int t = blockIdx.x, b = 0, r0 = -1, nrows = 0;
+  // find this block's tile: tiles of ROWS rows, counted sequence by sequence.  Blocks are taken from
+  // the back: a sequence's late tiles see the most keys and should start first.
+  int t = gridDim.x - 1 - blockIdx.x, b = 0, r0 = -1, nrows = 0;
   for (; b < a.batch; ++b) {
     const int begin = a.cu_rows[b], n = a.cu_rows[b + 1] - begin;
     const int tiles = (n + ROWS - 1) / ROWS;
@@ -372,7 +373,6 @@ __global__ __launch_bounds__(NW * 64) void attn_rows_kernel(AttnArgs a, int head
     unsigned char* cur = smem + ((lb - blk_first) & 1) * L::STAGE;
     unsigned char* nxt = smem + ((lb - blk_first + 1) & 1) * L::STAGE;
     const bool more = lb < blk_last;
-    if (more) fetch(lb + 1);  // in flight while this block is multiplied
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int t0 = lb * BS + half * 32;
@@ -415,7 +415,14 @@ __global__ __launch_bounds__(NW * 64) void attn_rows_kernel(AttnArgs a, int head
         }
       }
     }
-    if (more) stash(lb + 1, nxt);  // nobody reads nxt: its last readers passed the barrier below one round ago
+    // The next block is copied after this one's products: its registers are then not live across them,
+    // which keeps a wave within half the register file, and the copy's latency is covered by the
+    // other block resident on the compute unit.  Nobody reads nxt: its last readers passed the
+    // barrier below one round ago.
+    if (more) {
+      fetch(lb + 1);
+      stash(lb + 1, nxt);
+    }
     __syncthreads();
   }
 #pragma unroll

@@ -61,7 +61,7 @@ constexpr int TBK = 64;           // k per stage
 constexpr int TLD = TBK + 8;      // padded LDS row, in elements (144 bytes: conflict-free b128 reads)
 
 template <int WM, int WN, int EPI, typename TO>
-__global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A, int lda,
+__global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A, int lda,
                                                               const bf16_t* __restrict__ W, int ldw,
                                                               TO* __restrict__ C, int ldc, int M, int N,
                                                               int K, int tiles_m, int tiles_n) {
@@ -284,77 +284,94 @@ int launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, in
 // 16 columns.  The block's KW waves own contiguous K slices and keep their x fragments in
 // registers across the tiles, so x is read once per block and each tile costs weight loads only
 // (all of a tile's loads are in flight together).  Partial tiles meet in LDS, summed in wave order.
-constexpr int V3_KB = 8;    // k-steps (of 32) whose x fragments a wave holds at a time
+// Up to 64 rows: MT row tiles of 16 share every weight fragment.
 constexpr int V3_MAXT = 8;  // tiles a block may own
+// k-steps (of 32) whose x fragments a wave holds at a time, and waves per block: both shrink as the
+// row tiles (each with x fragments and accumulators of its own) grow
+constexpr int v3_kb(int mt) { return mt <= 2 ? 8 / mt : 2; }
+constexpr int v3_kw(int mt) { return mt == 1 ? 16 : 8; }
 
-template <int KW, int EPI, typename TO>
+template <int KW, int MT, int EPI, typename TO>
 __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16_t* __restrict__ X, int ldx,
                                                                       const bf16_t* __restrict__ W, int ldw,
                                                                       TO* __restrict__ C, int ldc, int M, int N,
                                                                       int K, int cols_per_block, int ks_per_wave) {
-  __shared__ float red[2][KW][256];
+  constexpr int KB = v3_kb(MT);
+  constexpr int NBUF = MT == 1 ? 2 : 1;
+  constexpr int VALS = MT * 4;  // accumulator values a lane holds per tile
+  __shared__ float red[NBUF][KW][VALS * 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, c16 = lane & 15;
   const int col_begin = blockIdx.x * cols_per_block;
   const int col_end = min(N, col_begin + cols_per_block);
   if (col_begin >= N) return;
   const int ntiles = (col_end - col_begin + 15) / 16;
-  const int k_wave = wave * ks_per_wave * 32;                 // this wave's slice [k_wave, k_stop)
+  const int k_wave = wave * ks_per_wave * 32;  // this wave's slice [k_wave, k_stop)
   const int k_stop = min(K, k_wave + ks_per_wave * 32);
-  const bf16_t* xp = X + (long long)min(c16, M - 1) * ldx;  // k below already holds the lane's g * 8
+  const bf16_t* xp[MT];  // k below already holds the lane's g * 8
+#pragma unroll
+  for (int m = 0; m < MT; ++m) xp[m] = X + (long long)min(m * 16 + c16, M - 1) * ldx;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
-  f32x4 acc[V3_MAXT];
+  f32x4 acc[V3_MAXT][MT];
 #pragma unroll
-  for (int t = 0; t < V3_MAXT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < V3_MAXT; ++t)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[t][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  for (int kb = k_wave; kb < k_stop; kb += V3_KB * 32) {
-    u32x4 xv[V3_KB];
+  for (int kb = k_wave; kb < k_stop; kb += KB * 32) {
+    u32x4 xv[KB][MT];
 #pragma unroll
-    for (int s = 0; s < V3_KB; ++s) {
+    for (int s = 0; s < KB; ++s) {
       const int k = kb + s * 32 + g * 8;
-      xv[s] = (k < k_stop) ? *(const u32x4*)(xp + k) : zero;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) xv[s][m] = (k < k_stop) ? *(const u32x4*)(xp[m] + k) : zero;
     }
 #pragma unroll
     for (int t = 0; t < V3_MAXT; ++t) {
       if (t < ntiles) {
         const int nrow = min(col_begin + t * 16 + c16, col_end - 1);
         const bf16_t* wp = W + (long long)nrow * ldw;
-        u32x4 wv[V3_KB];
+        u32x4 wv[KB];
 #pragma unroll
-        for (int s = 0; s < V3_KB; ++s) {
+        for (int s = 0; s < KB; ++s) {
           const int k = kb + s * 32 + g * 8;
           wv[s] = (k < k_stop) ? *(const u32x4*)(wp + k) : zero;
         }
 #pragma unroll
-        for (int s = 0; s < V3_KB; ++s)
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[s]), as_bf16x8(wv[s]), acc[t], 0, 0, 0);
+        for (int s = 0; s < KB; ++s)
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xv[s][m]), as_bf16x8(wv[s]), acc[t][m],
+                                                                0, 0, 0);
       }
     }
   }
-  // acc[t][e] = C[(lane / 16) * 4 + e][col_begin + 16 t + lane % 16], partial over this wave's k
+  // acc[t][m][e] = C[m * 16 + (lane / 16) * 4 + e][col_begin + 16 t + lane % 16], partial over this
+  // wave's k.  The waves share out the (m, e) values of a tile and each sums its share over all waves,
+  // in wave order.
 #pragma unroll
   for (int t = 0; t < V3_MAXT; ++t) {
     if (t < ntiles) {
-      float(*r)[256] = red[t & 1];
+      float(*r)[VALS * 64] = red[NBUF == 2 ? (t & 1) : 0];
+      if (NBUF == 1 && t > 0) __syncthreads();  // the tile before has been read
 #pragma unroll
-      for (int e = 0; e < 4; ++e) r[wave][e * 64 + lane] = acc[t][e];
-      __syncthreads();  // also: the buffer written two tiles ago has been read by then
-      if (wave == t % KW) {
-        const int col = col_begin + t * 16 + c16;
+      for (int m = 0; m < MT; ++m)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float s = 0.f;
+        for (int e = 0; e < 4; ++e) r[wave][(m * 4 + e) * 64 + lane] = acc[t][m][e];
+      __syncthreads();  // with two buffers also: the buffer written two tiles ago has been read by then
+      const int col = col_begin + t * 16 + c16;
+      for (int v = (wave + t) % KW; v < VALS; v += KW) {
+        float s = 0.f;
 #pragma unroll
-          for (int w = 0; w < KW; ++w) s += r[w][e * 64 + lane];
-          const int row = g * 4 + e;
-          if (EPI == EPI_SWIGLU) {
-            const float up = __shfl(s, lane + 8, 64);
-            if (c16 < 8 && row < M && col + 8 < col_end)
-              store_out<TO>(C + (long long)row * ldc + ((col_begin + t * 16) >> 1) + c16, silu_mul(s, up));
-          } else {
-            if (row < M && col < col_end) store_out<TO>(C + (long long)row * ldc + col, s);
-          }
+        for (int w = 0; w < KW; ++w) s += r[w][v * 64 + lane];
+        const int row = (v >> 2) * 16 + g * 4 + (v & 3);
+        if (EPI == EPI_SWIGLU) {
+          const float up = __shfl(s, lane + 8, 64);
+          if (c16 < 8 && row < M && col + 8 < col_end)
+            store_out<TO>(C + (long long)row * ldc + ((col_begin + t * 16) >> 1) + c16, silu_mul(s, up));
+        } else {
+          if (row < M && col < col_end) store_out<TO>(C + (long long)row * ldc + col, s);
         }
       }
     }
@@ -373,10 +390,10 @@ static int lq_compute_units() {
   return n;
 }
 
-template <int EPI, typename TO>
+template <int MT, int EPI, typename TO>
 int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc,
                      hipStream_t stream) {
-  constexpr int KW = 16;
+  constexpr int KW = v3_kw(MT);
   const int cus = lq_compute_units();
   // equal runs of columns, in units of 16 (8 without the paired epilogue), at most V3_MAXT tiles each
   const int unit = EPI == EPI_SWIGLU ? 16 : 8;
@@ -389,7 +406,7 @@ int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K,
   const int grid = lq_ceil_div(N, cols);
   const int ksteps = lq_ceil_div(K, 32);
   const int ks_per_wave = lq_ceil_div(ksteps, KW);
-  gemm_bf16_skinny_v3_kernel<KW, EPI, TO><<<grid, KW * 64, 0, stream>>>(
+  gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO><<<grid, KW * 64, 0, stream>>>(
       (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, cols, ks_per_wave);
   LQ_CHECK_LAUNCH("linear(mfma skinny v3)");
   return 0;
@@ -411,17 +428,40 @@ int pick_skinny(const void* x, const void* w, void* out, int M, int N, int K, in
 template <int EPI, typename TO>
 int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
              hipStream_t stream) {
+  // wide enough to give every compute unit a run of columns: the balanced kernel; else the simple one
+  const bool wide = N >= 8 * lq_compute_units() && K >= 512;
   if (M <= 16) {
-    // wide enough to give every compute unit a run of columns: the balanced kernel; else the simple one
-    if (N >= 8 * lq_compute_units() && K >= 512) return launch_skinny_v3<EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (wide) return launch_skinny_v3<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
     return pick_skinny<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
-  if (M <= 32) return pick_skinny<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-  if (M <= 64) return pick_skinny<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  if (M <= 32) {
+    if (wide) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    return pick_skinny<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  }
+  if (M <= 64) {
+    if (wide) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    return pick_skinny<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  }
+  // the wider tile reuses each x fragment for twice the columns; it pays once there are enough tiles
+  // of it to fill every compute unit twice over
+  const long long wide_tiles = (long long)lq_ceil_div(M, 128) * lq_ceil_div(N, 256);
+  if (wide_tiles >= 2 * lq_compute_units()) return launch_tiled<2, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   return launch_tiled<2, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
 }
 
 }  // namespace
+
+// Tuning hook: the tiled kernel with a given wave tile (float32 out, no epilogue).
+extern "C" int lq_debug_gemm_tiled(const void* x, const void* w, void* out, int M, int N, int K, int wm, int wn,
+                                   hipStream_t stream) {
+  if (wm == 2 && wn == 2) return launch_tiled<2, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
+  if (wm == 4 && wn == 2) return launch_tiled<4, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
+  if (wm == 2 && wn == 4) return launch_tiled<2, 4, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
+  if (wm == 4 && wn == 4) return launch_tiled<4, 4, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
+  if (wm == 1 && wn == 2) return launch_tiled<1, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
+  lq_set_error("no such tile");
+  return -1;
+}
 
 // Whether the MFMA kernels take this problem (the caller falls back to the generic kernel if not).
 bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int lda, int ldw) {
