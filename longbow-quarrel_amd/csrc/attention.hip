@@ -13,7 +13,8 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
                       int hd, const int* row_pos, const int* seq_slot, const int* cu_rows,
                       const int* block_table, int bt_stride, const void* kcache, const void* vcache,
                       float scale, int window, int decode, int max_len, float* workspace,
-                      long long workspace_floats, hipStream_t stream);
+                      long long workspace_floats, const void* k_new, const void* v_new, int ldk, int ldv,
+                      const float* cs, hipStream_t stream);
 
 // Floats of workspace lq_attention wants for this launch (0: none).
 extern "C" long long lq_attention_workspace(int dtype, int rows, int nh, int nkv, int hd, int block_size,
@@ -23,6 +24,12 @@ extern "C" long long lq_attention_workspace(int dtype, int rows, int nh, int nkv
   return lq_attention_mfma_workspace(rows, nh, hd, max_len);
 }
 
+// Whether a decoding launch can take the rotation of q and k and the cache write upon itself
+// (lq_attention with k_new, v_new and a cos/sin table; q, k, v are then the unrotated projections).
+extern "C" int lq_attention_folds_rope(int dtype, int nh, int nkv, int hd, int block_size) {
+  return hd % 64 == 0 && lq_attention_mfma_accepts(dtype, nh, nkv, hd, block_size, 8, 8, nullptr, nullptr, 1);
+}
+
 // `decode` != 0 promises one row per sequence; `max_len` is then an upper bound of the
 // sequences' lengths after this step (it sizes the split grid, not the result).
 extern "C" int lq_attention(const void* q, int ldq, void* out, int ldo, int dtype, int rows, int batch,
@@ -30,7 +37,8 @@ extern "C" int lq_attention(const void* q, int ldq, void* out, int ldo, int dtyp
                             const int* seq_slot, const int* cu_rows, const int* block_table,
                             int bt_stride, const void* kcache, const void* vcache, int block_size,
                             float scale, int window, int decode, int max_len, float* workspace,
-                            long long workspace_floats, int force_generic, hipStream_t stream) {
+                            long long workspace_floats, const void* k_new, const void* v_new, int ldk, int ldv,
+                            const float* cs, int force_generic, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && batch > 0, "attention: rows %d and sequences %d must be positive", rows, batch);
   LQ_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "attention: %d heads over %d kv heads", nh, nkv);
   LQ_REQUIRE(hd > 0 && block_size > 0 && bt_stride > 0, "attention: bad sizes");
@@ -41,7 +49,8 @@ extern "C" int lq_attention(const void* q, int ldq, void* out, int ldo, int dtyp
   if (!force_generic && lq_attention_mfma_accepts(dtype, nh, nkv, hd, block_size, ldq, ldo, q, out, decode))
     return lq_attention_mfma(q, ldq, out, ldo, rows, batch, nh, nkv, hd, row_pos, seq_slot, cu_rows,
                              block_table, bt_stride, kcache, vcache, scale, window, decode, max_len,
-                             workspace, workspace_floats, stream);
+                             workspace, workspace_floats, k_new, v_new, ldk, ldv, cs, stream);
+  LQ_REQUIRE(cs == nullptr, "attention: the folded rotation was asked of a launch the matrix-core kernel does not take");
   return lq_attention_generic(q, ldq, out, ldo, dtype, rows, nh, nkv, hd, row_pos, row_seq, seq_slot,
                               block_table, bt_stride, kcache, vcache, block_size, scale, window, stream);
 }

@@ -127,6 +127,12 @@ struct AttnArgs {
   float* part_o;   // [rows][nh][nsplit][HD]
   float* part_ml;  // [rows][nh][nsplit][2]
   int nsplit;
+  // decode with the rotation and the cache write folded in (all null otherwise): the step's
+  // unrotated keys and values, and cos/sin of every row's angles [rows][HD/2][2]
+  const bf16_t* k_new;
+  const bf16_t* v_new;
+  int ldk, ldv;
+  const float* cs;
 };
 
 // One chunk's operands as they come from memory: 16 bytes a lane for each K fragment, two 8-byte
@@ -494,11 +500,54 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
   w.first_key[0] = lo;
   w.free_to[0] = -1;  // columns beyond the group's heads are never valid: always the masked path
   w.free_from[0] = 0;
+  u32x4 qraw[HD / 32];
   {
     const bf16_t* qr = a.q + (long long)r * a.ldq + h * HD + g * 8;
 #pragma unroll
-    for (int kk = 0; kk < HD / 32; ++kk) w.q[0][kk] = as_bf16x8(*(const u32x4*)(qr + kk * 32));
+    for (int kk = 0; kk < HD / 32; ++kk) qraw[kk] = *(const u32x4*)(qr + kk * 32);
   }
+  if (HD % 64 == 0 && a.cs != nullptr) {
+    // The rotation and the cache write of this step, folded in.  Pair (i, i + HD/2): a lane's
+    // fragment kk holds i = kk*32 + (lane/16)*8 + j and its fragment kk + HD/64 the partners.
+    const float* cs = a.cs + (long long)r * HD;  // [HD/2][2]
+#pragma unroll
+    for (int kk = 0; kk < HD / 64; ++kk) {
+      const int i0 = kk * 32 + g * 8;
+      u32x4 lo4 = qraw[kk], hi4 = qraw[kk + HD / 64];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f32x4 c2 = *(const f32x4*)(cs + (i0 + 2 * j) * 2);  // cos, sin of i0+2j and of i0+2j+1
+        const float x0a = __uint_as_float(lo4[j] << 16), x0b = __uint_as_float(lo4[j] & 0xffff0000u);
+        const float x1a = __uint_as_float(hi4[j] << 16), x1b = __uint_as_float(hi4[j] & 0xffff0000u);
+        lo4[j] = pack_bf16(x0a * c2[0] - x1a * c2[1], x0b * c2[2] - x1b * c2[3]);
+        hi4[j] = pack_bf16(x0a * c2[1] + x1a * c2[0], x0b * c2[3] + x1b * c2[2]);
+      }
+      qraw[kk] = lo4;
+      qraw[kk + HD / 64] = hi4;
+    }
+    // the block whose split holds position p writes the row's rotated key and its value
+    if (split == p / SPLIT) {
+      const long long blk = table[p / BS];
+      const int off = p % BS;
+      const bf16_t* kr = a.k_new + (long long)r * a.ldk + kvh * HD;
+      const bf16_t* vr = a.v_new + (long long)r * a.ldv + kvh * HD;
+      bf16_t* kdst = const_cast<bf16_t*>(a.kcache) + ((blk * a.nkv + kvh) * BS + off) * (long long)HD;
+      bf16_t* vdst = const_cast<bf16_t*>(a.vcache) + ((blk * a.nkv + kvh) * (long long)HD) * BS + off;
+      for (int i = threadIdx.x; i < HD / 2; i += NW * 64) {
+        const float x0 = bf16_to_f32(kr[i]), x1 = bf16_to_f32(kr[i + HD / 2]);
+        const float c = cs[2 * i], sn = cs[2 * i + 1];
+        bf16_t r0, r1;
+        r0.bits = (uint16_t)(pack_bf16(x0 * c - x1 * sn, 0.f) & 0xffffu);
+        r1.bits = (uint16_t)(pack_bf16(x0 * sn + x1 * c, 0.f) & 0xffffu);
+        kdst[i] = r0;
+        kdst[i + HD / 2] = r1;
+      }
+      for (int d = threadIdx.x; d < HD; d += NW * 64) vdst[(long long)d * BS] = vr[d];
+    }
+    __syncthreads();  // the block's own stores are visible to its loads below
+  }
+#pragma unroll
+  for (int kk = 0; kk < HD / 32; ++kk) w.q[0][kk] = as_bf16x8(qraw[kk]);
   // chunk numbering is absolute within the split, so that a wave's chunks depend on positions only
   int t_first = split * SPLIT + wave * 32;
   while (t_first < s_begin) t_first += NW * 32;
@@ -635,7 +684,8 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
                       int hd, const int* row_pos, const int* seq_slot, const int* cu_rows,
                       const int* block_table, int bt_stride, const void* kcache, const void* vcache,
                       float scale, int window, int decode, int max_len, float* workspace,
-                      long long workspace_floats, hipStream_t stream) {
+                      long long workspace_floats, const void* k_new, const void* v_new, int ldk, int ldv,
+                      const float* cs, hipStream_t stream) {
   AttnArgs a;
   a.q = (const bf16_t*)q;
   a.ldq = ldq;
@@ -656,6 +706,16 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
   a.part_o = nullptr;
   a.part_ml = nullptr;
   a.nsplit = 1;
+  a.k_new = (const bf16_t*)k_new;
+  a.v_new = (const bf16_t*)v_new;
+  a.ldk = ldk;
+  a.ldv = ldv;
+  a.cs = cs;
+  if (cs != nullptr) {
+    LQ_REQUIRE(decode && hd % 64 == 0 && k_new && v_new && ldk >= nkv * hd && ldv >= nkv * hd,
+               "attention: the folded rotation needs a decoding step, a head size that is a multiple of 64 and the step's keys and values");
+    LQ_REQUIRE(((uintptr_t)cs % 16) == 0, "attention: the cos/sin table must be 16-byte aligned");
+  }
   if (decode) {
     LQ_REQUIRE(rows == batch, "attention: decoding needs one row a sequence (%d rows, %d sequences)", rows, batch);
     LQ_REQUIRE(max_len > 0, "attention: decoding needs the longest sequence length");

@@ -379,3 +379,30 @@ extern "C" int lq_rope_store(void* q, const void* k, const void* v, int dtype, i
   LQ_CHECK_LAUNCH("rope_store");
   return 0;
 }
+
+// ---------------------------------------------------------------- cos/sin table of a step
+// cs[r][i] = (cos, sin) of row_pos[r] * f_i, angles formed and reduced in double as in rope_store.
+// Positions are the same for every layer of a step, so one launch serves them all.
+__global__ void rope_table_kernel(const double* __restrict__ freqs, const int* __restrict__ row_pos,
+                                  float* __restrict__ cs, int half) {
+  const int r = blockIdx.x;
+  const int p = row_pos[r];
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const double a = (double)p * freqs[i];
+    const double n = rint(a * 0.15915494309189533577);
+    double rem = fma(-n, 6.283185307179586232, a);
+    rem = fma(-n, 2.4492935982947064e-16, rem);
+    float sn, c;
+    sincosf((float)rem, &sn, &c);
+    cs[((long long)r * half + i) * 2] = c;
+    cs[((long long)r * half + i) * 2 + 1] = sn;
+  }
+}
+
+extern "C" int lq_rope_table(const double* freqs, const int* row_pos, float* cs, int rows, int half,
+                             hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && half > 0, "rope_table: rows %d and pairs %d must be positive", rows, half);
+  rope_table_kernel<<<rows, 64, 0, stream>>>(freqs, row_pos, cs, half);
+  LQ_CHECK_LAUNCH("rope_table");
+  return 0;
+}

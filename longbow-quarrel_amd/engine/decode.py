@@ -100,10 +100,14 @@ class DecodeGraph:
         """Runs the body's allocations without launching, to learn the workspace size."""
         e = self.engine
 
+        queries = ("attention_workspace", "attention_folds_rope", "linear_swiglu_supported")
+
         class _Null:
+            """Answers the size and capability questions truthfully, launches nothing."""
+
             def __getattr__(self, name):
-                if name == "attention_workspace":
-                    return e.kernels.attention_workspace
+                if name in queries:
+                    return getattr(e.kernels, name)
                 return lambda *a, **k: None
 
         ctx = self.context()

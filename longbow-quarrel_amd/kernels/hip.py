@@ -278,15 +278,36 @@ class HipKernels:
                                                    c_int(kv_heads), c_int(head_dim), c_int(block_size),
                                                    c_int(1 if decode else 0), c_int(max_len)))
 
+    def attention_folds_rope(self, dtype: torch.dtype, heads: int, kv_heads: int, head_dim: int, block_size: int) -> bool:
+        """Whether a decoding `attention` launch can rotate q and k and write the cache itself."""
+        if self.force_generic or dtype not in _DTYPE_CODE:
+            return False
+        return bool(self.lib.lq_attention_folds_rope(c_int(_DTYPE_CODE[dtype]), c_int(heads), c_int(kv_heads),
+                                                     c_int(head_dim), c_int(block_size)))
+
+    def rope_table(self, freqs: torch.Tensor, row_pos: torch.Tensor, out: torch.Tensor) -> None:
+        """out[r, i] = (cos, sin) of row_pos[r] * freqs[i]; float32 [rows, pairs, 2]."""
+        self._dev(freqs, row_pos, out)
+        rows, half = out.shape[0], out.shape[1]
+        self._i32(row_pos, "row_pos", rows)
+        if freqs.dtype != torch.float64 or freqs.numel() != half or out.dtype != torch.float32 \
+                or tuple(out.shape) != (rows, half, 2) or not out.is_contiguous():
+            raise KernelLibraryError("rope_table: freqs float64 [pairs], out dense float32 [rows, pairs, 2]")
+        self._check(self.lib.lq_rope_table(_ptr(freqs), _ptr(row_pos), _ptr(out), c_int(rows), c_int(half), self.stream))
+
     def attention(self, q: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
                   row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor, cu_rows: torch.Tensor,
                   block_table: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                   block_size: int, scale: float, window: int = 0, decode: bool = False, max_len: int = 0,
-                  workspace: Optional[torch.Tensor] = None) -> None:
+                  workspace: Optional[torch.Tensor] = None, k_new: Optional[torch.Tensor] = None,
+                  v_new: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None) -> None:
         """Causal grouped-query attention of the step's rows over their slots' cached keys.
 
         `decode` promises one row per sequence; `max_len` is then an upper bound of the lengths
-        after this step and `workspace` float32 scratch of `attention_workspace(...)` entries."""
+        after this step and `workspace` float32 scratch of `attention_workspace(...)` entries.
+        With `cos_sin` (a `rope_table` of this step; only where `attention_folds_rope` says so) q, k_new
+        and v_new are the unrotated projections: the launch rotates q and k and writes k and v into
+        the cache itself."""
         self._dev(q, out, row_pos, row_seq, seq_slot, cu_rows, block_table, kcache, vcache, workspace)
         rows = q.shape[0]
         batch = seq_slot.numel()
@@ -311,13 +332,26 @@ class HipKernels:
             if workspace.dtype != torch.float32 or not workspace.is_contiguous():
                 raise KernelLibraryError("attention: workspace must be dense float32")
             ws_n = workspace.numel()
+        ldk = ldv = 0
+        if cos_sin is not None:
+            self._dev(k_new, v_new, cos_sin)
+            if k_new is None or v_new is None or not decode:
+                raise KernelLibraryError("attention: the folded rotation needs the step's keys and values and a decoding step")
+            if k_new.dtype != q.dtype or v_new.dtype != q.dtype or k_new.shape[0] != rows or v_new.shape[0] != rows \
+                    or k_new.shape[1] < kv_heads * head_dim or v_new.shape[1] < kv_heads * head_dim:
+                raise KernelLibraryError("attention: k_new / v_new do not match the rows or the kv width")
+            if cos_sin.dtype != torch.float32 or tuple(cos_sin.shape) != (rows, head_dim // 2, 2) or not cos_sin.is_contiguous():
+                raise KernelLibraryError("attention: cos_sin must be dense float32 [rows, head_dim/2, 2]")
+            ldk, ldv = self._rows2d(k_new, "k_new"), self._rows2d(v_new, "v_new")
         self._check(self.lib.lq_attention(
             _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")),
             c_int(_code(q)), c_int(rows), c_int(batch), c_int(heads), c_int(kv_heads), c_int(head_dim),
             _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(cu_rows), _ptr(block_table),
             c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
             c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
-            c_longlong(ws_n), c_int(1 if self.force_generic else 0), self.stream))
+            c_longlong(ws_n), _ptr(k_new if cos_sin is not None else None),
+            _ptr(v_new if cos_sin is not None else None), c_int(ldk), c_int(ldv), _ptr(cos_sin),
+            c_int(1 if self.force_generic else 0), self.stream))
 
     # ------------------------------------------------------------------ sampling
     def apply_penalty(self, logits: torch.Tensor, seq_slot: torch.Tensor, recent: torch.Tensor,

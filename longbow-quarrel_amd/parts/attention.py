@@ -75,20 +75,30 @@ class GQAttention(Mixer):
         k = qkv[:, self.q_width : self.q_width + self.kv_width]
         v = qkv[:, self.q_width + self.kv_width :]
         freqs = self.position.rotary_frequencies
-        if freqs is None:
-            self.position.apply(q, k, ctx)
-        if cache.write:
-            kn.rope_store(q, k, v, self.heads, self.kv_heads, self.head_dim, freqs, ctx.row_pos,
-                          ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size)
-        elif freqs is not None:
-            kn.rope_store(q, None, None, self.heads, 0, self.head_dim, freqs, ctx.row_pos)
         att = ctx.ws.alloc((rows, self.q_width), ctx.dtype)
         need = kn.attention_workspace(ctx.dtype, rows, self.heads, self.kv_heads, self.head_dim,
                                       cache.block_size, ctx.decode, ctx.max_len)
         scratch = ctx.ws.alloc((need,), torch.float32) if need else None
-        kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
-                     ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
-                     self.scale, self.window, decode=ctx.decode, max_len=ctx.max_len, workspace=scratch)
+        # a decoding step can leave the rotation and the cache write to the attention kernel itself
+        folded = (ctx.decode and cache.write and freqs is not None and hasattr(self.position, "cos_sin")
+                  and getattr(kn, "attention_folds_rope", lambda *a: False)(
+                      ctx.dtype, self.heads, self.kv_heads, self.head_dim, cache.block_size))
+        if folded:
+            kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
+                         ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
+                         self.scale, self.window, decode=True, max_len=ctx.max_len, workspace=scratch,
+                         k_new=k, v_new=v, cos_sin=self.position.cos_sin(ctx))
+        else:
+            if freqs is None:
+                self.position.apply(q, k, ctx)
+            if cache.write:
+                kn.rope_store(q, k, v, self.heads, self.kv_heads, self.head_dim, freqs, ctx.row_pos,
+                              ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size)
+            elif freqs is not None:
+                kn.rope_store(q, None, None, self.heads, 0, self.head_dim, freqs, ctx.row_pos)
+            kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
+                         ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
+                         self.scale, self.window, decode=ctx.decode, max_len=ctx.max_len, workspace=scratch)
         out = ctx.ws.alloc((rows, self.width), torch.float32)
         project(kn, ctx, att, self.w_o, out)
         return out

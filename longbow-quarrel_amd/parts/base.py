@@ -186,6 +186,7 @@ class StepContext:
     max_len: int = 0
     decode: bool = False  # every sequence brings exactly one token
     logits_out: Optional[torch.Tensor] = None  # where the logits go (a captured step's fixed buffer)
+    shared: Dict[Any, Any] = field(default_factory=dict)  # what parts compute once a step and share
 
 
 @dataclass

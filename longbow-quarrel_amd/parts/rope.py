@@ -55,6 +55,17 @@ class RotaryEncoding(PositionEncoding):
         super().bind(tensors, env)
         self.rotary_frequencies = torch.tensor(self.table, dtype=torch.float64, device=env.device)
 
+    def cos_sin(self, ctx: StepContext) -> torch.Tensor:
+        """cos and sin of every row's angles, float32 [rows, head_dim/2, 2]: the same for every layer
+        of a step that rotates with these frequencies, so it is computed once and shared."""
+        key = ("rope_cos_sin", tuple(self.table))
+        table = ctx.shared.get(key)
+        if table is None:
+            table = ctx.ws.alloc((ctx.rows, self.head_dim // 2, 2), torch.float32)
+            ctx.kernels.rope_table(self.rotary_frequencies, ctx.row_pos, table)
+            ctx.shared[key] = table
+        return table
+
     def apply(self, q: torch.Tensor, k: torch.Tensor, ctx: StepContext) -> None:
         heads = q.shape[1] // self.head_dim
         kv_heads = k.shape[1] // self.head_dim

@@ -326,3 +326,45 @@ def test_linear_with_fused_swiglu(kn, m, inner, k):
     out32 = torch.empty((m, inner), dtype=torch.float32, device=DEV)
     kn.linear_swiglu(x, w, out32)
     assert rel_err(out32, want) < 2e-5
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(32, 8, 128), (4, 2, 64), (16, 1, 64), (6, 3, 192)])
+@pytest.mark.parametrize("window", [0, 100])
+def test_decode_attention_with_rotation_and_cache_write_folded_in(kn, heads, kv_heads, head_dim, window):
+    """One launch that rotates q and k, writes k and v into the cache and attends, against the two
+    separate kernels (rope_store, then attention)."""
+    dtype = torch.bfloat16
+    lengths = [700, 64, 257, 1, 1300]
+    assert kn.attention_folds_rope(dtype, heads, kv_heads, head_dim, BS)
+    kc, vc, table, slots, dense = paged_cache(lengths, kv_heads, head_dim, dtype, 51)
+    kc2, vc2 = kc.clone(), vc.clone()
+    rows = len(lengths)
+    width = (heads + 2 * kv_heads) * head_dim
+    qkv = rnd((rows, width), 52, dtype)
+    qkv2 = qkv.clone()
+    pos = [n - 1 for n in lengths]
+    freqs = plain.rope_frequencies(head_dim, 500000.0).to(DEV)
+    cu = list(range(rows + 1))
+    scale = 1.0 / math.sqrt(head_dim)
+    need = kn.attention_workspace(dtype, rows, heads, kv_heads, head_dim, BS, True, max(lengths))
+    ws = torch.empty(max(need, 1), dtype=torch.float32, device=DEV)
+
+    def views(t):
+        return t[:, : heads * head_dim], t[:, heads * head_dim : (heads + kv_heads) * head_dim], t[:, (heads + kv_heads) * head_dim :]
+
+    q, k, v = views(qkv)
+    out_a = torch.empty((rows, heads * head_dim), dtype=dtype, device=DEV)
+    kn.rope_store(q, k, v, heads, kv_heads, head_dim, freqs, i32(pos), i32(range(rows)), i32(slots), table, kc, vc, BS)
+    kn.attention(q, out_a, heads, kv_heads, head_dim, i32(pos), i32(range(rows)), i32(slots), i32(cu), table, kc, vc, BS,
+                 scale, window, decode=True, max_len=max(lengths), workspace=ws)
+    q2, k2, v2 = views(qkv2)
+    cs = torch.empty((rows, head_dim // 2, 2), dtype=torch.float32, device=DEV)
+    kn.rope_table(freqs, i32(pos), cs)
+    ang = torch.tensor(pos, dtype=torch.float64)[:, None] * freqs.cpu()[None, :]
+    assert float((cs[..., 0].cpu().double() - torch.cos(ang)).abs().max()) < 1e-6
+    assert float((cs[..., 1].cpu().double() - torch.sin(ang)).abs().max()) < 1e-6
+    out_b = torch.empty_like(out_a)
+    kn.attention(q2, out_b, heads, kv_heads, head_dim, i32(pos), i32(range(rows)), i32(slots), i32(cu), table, kc2, vc2,
+                 BS, scale, window, decode=True, max_len=max(lengths), workspace=ws, k_new=k2, v_new=v2, cos_sin=cs)
+    assert torch.equal(kc, kc2) and torch.equal(vc, vc2)  # the same rows of the cache were written, with the same bits
+    assert rel_err(out_b, out_a.double().cpu()) < 4e-3
