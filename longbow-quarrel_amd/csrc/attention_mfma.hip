@@ -482,7 +482,7 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
   float* lds_l = lds_m + NW * G;         // [NW][G]
   const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, g = lane >> 4;
-  const int r = a.cu_rows[b];
+  const int r = b;  // a decoding step has one row a sequence, in the order of the sequences
   const int p = a.row_pos[r];
   const int lo = (a.window > 0 && p >= a.window) ? p - a.window + 1 : 0;
   const int s_begin = max(split * SPLIT, (lo / 32) * 32);
@@ -525,15 +525,17 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
       qraw[kk] = lo4;
       qraw[kk + HD / 64] = hi4;
     }
-    // the block whose split holds position p writes the row's rotated key and its value
-    if (split == p / SPLIT) {
+    // The wave that will read the chunk holding position p writes the row's rotated key and its
+    // value there first; a workgroup-scope fence orders its lanes' stores before its lanes' loads.
+    // No other wave (and no other block) reads that chunk.
+    if (split == p / SPLIT && wave == ((p - split * SPLIT) / 32) % NW) {
       const long long blk = table[p / BS];
       const int off = p % BS;
       const bf16_t* kr = a.k_new + (long long)r * a.ldk + kvh * HD;
       const bf16_t* vr = a.v_new + (long long)r * a.ldv + kvh * HD;
       bf16_t* kdst = const_cast<bf16_t*>(a.kcache) + ((blk * a.nkv + kvh) * BS + off) * (long long)HD;
       bf16_t* vdst = const_cast<bf16_t*>(a.vcache) + ((blk * a.nkv + kvh) * (long long)HD) * BS + off;
-      for (int i = threadIdx.x; i < HD / 2; i += NW * 64) {
+      for (int i = lane; i < HD / 2; i += 64) {
         const float x0 = bf16_to_f32(kr[i]), x1 = bf16_to_f32(kr[i + HD / 2]);
         const float c = cs[2 * i], sn = cs[2 * i + 1];
         bf16_t r0, r1;
@@ -542,9 +544,9 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
         kdst[i] = r0;
         kdst[i + HD / 2] = r1;
       }
-      for (int d = threadIdx.x; d < HD; d += NW * 64) vdst[(long long)d * BS] = vr[d];
+      for (int d = lane; d < HD; d += 64) vdst[(long long)d * BS] = vr[d];
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
     }
-    __syncthreads();  // the block's own stores are visible to its loads below
   }
 #pragma unroll
   for (int kk = 0; kk < HD / 32; ++kk) w.q[0][kk] = as_bf16x8(qraw[kk]);
@@ -602,7 +604,7 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
 template <int HD>
 __global__ __launch_bounds__(64) void attn_merge_kernel(AttnArgs a) {
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int r = a.cu_rows[b];
+  const int r = b;
   const int p = a.row_pos[r];
   const int lo = (a.window > 0 && p >= a.window) ? p - a.window + 1 : 0;
   const int s_first = lo / SPLIT, s_last = p / SPLIT;
