@@ -33,16 +33,19 @@ extern "C" int lq_embed(const void* table, int table_dtype, const int* tokens, f
 // Per row: (x += delta, written back, if delta is given), s = sum x^2,
 // r = 1 / sqrt(s / D + eps), out = x * r * w.  eps inside the root, weight
 // after normalisation (internal/device/kernels.metal:905-942).
+// delta may come in `parts` pieces (the partial sums of a product whose K was split over blocks),
+// `part_stride` elements apart; they are added in ascending order.
 template <typename TD, typename TO, bool HAS_DELTA>
-__global__ void rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
-                               const float* __restrict__ w, TO* __restrict__ out, int D, float eps) {
+__global__ void rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int parts,
+                               long long part_stride, const float* __restrict__ w, TO* __restrict__ out, int D,
+                               float eps) {
   __shared__ float red[16];
   const long long base = (long long)blockIdx.x * D;
   float ss = 0.f;
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
     float v = x[base + j];
     if (HAS_DELTA) {
-      v += to_f32(delta[base + j]);
+      for (int s = 0; s < parts; ++s) v += to_f32(delta[s * part_stride + base + j]);
       x[base + j] = v;
     }
     ss += v * v;
@@ -80,6 +83,7 @@ __device__ inline void store4(bf16_t* p, f32x4_t v) {
 
 template <typename TD, typename TO, bool HAS_DELTA, int NV>
 __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                                           int parts, long long part_stride,
                                                            const float* __restrict__ w, TO* __restrict__ out,
                                                            int D, float eps) {
   __shared__ float red[16];
@@ -92,7 +96,7 @@ __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ x
     if (j < D) {
       v[i] = load4(x + base + j);
       if (HAS_DELTA) {
-        v[i] += load4(delta + base + j);
+        for (int s = 0; s < parts; ++s) v[i] += load4(delta + s * part_stride + base + j);
         store4(x + base + j, v[i]);
       }
       ss += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
@@ -108,14 +112,15 @@ __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ x
 }
 
 template <typename TD, typename TO, bool HAS>
-static void rmsnorm_launch(float* x, const void* delta, const float* w, void* out, int rows, int D, float eps,
-                           hipStream_t stream) {
+static void rmsnorm_launch(float* x, const void* delta, int parts, long long part_stride, const float* w, void* out,
+                           int rows, int D, float eps, hipStream_t stream) {
   const bool aligned = D % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
-                       ((uintptr_t)w % 16) == 0 && ((uintptr_t)delta % 16) == 0;
+                       ((uintptr_t)w % 16) == 0 && ((uintptr_t)delta % 16) == 0 && part_stride % 4 == 0;
   const int vecs = (D / 4 + 255) / 256;
   if (aligned && vecs <= 8) {
 #define LQ_REGS(NV) \
-  rmsnorm_regs_kernel<TD, TO, HAS, NV><<<rows, 256, 0, stream>>>(x, (const TD*)delta, w, (TO*)out, D, eps)
+  rmsnorm_regs_kernel<TD, TO, HAS, NV><<<rows, 256, 0, stream>>>(x, (const TD*)delta, parts, part_stride, w, \
+                                                                 (TO*)out, D, eps)
     if (vecs <= 1)
       LQ_REGS(1);
     else if (vecs <= 2)
@@ -128,14 +133,19 @@ static void rmsnorm_launch(float* x, const void* delta, const float* w, void* ou
     return;
   }
   const int threads = D >= 2048 ? 512 : (D >= 512 ? 256 : 64);
-  rmsnorm_kernel<TD, TO, HAS><<<rows, threads, 0, stream>>>(x, (const TD*)delta, w, (TO*)out, D, eps);
+  rmsnorm_kernel<TD, TO, HAS><<<rows, threads, 0, stream>>>(x, (const TD*)delta, parts, part_stride, w, (TO*)out, D,
+                                                            eps);
 }
 
-extern "C" int lq_rmsnorm(float* x, const void* delta, int delta_dtype, const float* w, float eps,
-                          void* out, int out_dtype, int rows, int D, hipStream_t stream) {
+extern "C" int lq_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, long long part_stride,
+                          const float* w, float eps, void* out, int out_dtype, int rows, int D,
+                          hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && D > 0, "rmsnorm: rows %d and width %d must be positive", rows, D);
+  LQ_REQUIRE(delta == nullptr || (parts >= 1 && (parts == 1 || part_stride >= (long long)rows * D)),
+             "rmsnorm: %d delta parts with stride %lld", parts, part_stride);
   LQ_REQUIRE(out_dtype == LQ_F32 || out_dtype == LQ_BF16, "rmsnorm: unknown out dtype %d", out_dtype);
-#define LQ_NORM_LAUNCH(TD, TO, HAS) rmsnorm_launch<TD, TO, HAS>(x, delta, w, out, rows, D, eps, stream)
+#define LQ_NORM_LAUNCH(TD, TO, HAS) \
+  rmsnorm_launch<TD, TO, HAS>(x, delta, parts, part_stride, w, out, rows, D, eps, stream)
   if (delta == nullptr) {
     if (out_dtype == LQ_F32)
       LQ_NORM_LAUNCH(float, float, false);
@@ -245,27 +255,29 @@ extern "C" int lq_swiglu(const void* gu, int in_dtype, void* out, int out_dtype,
 // out[i, :] = x[rows[i], :] (+ delta[rows[i], :]); picks the rows whose logits
 // are wanted before the final norm, carrying a not yet applied residual delta.
 template <typename TD, bool HAS_DELTA>
-__global__ void gather_rows_kernel(const float* __restrict__ x, const TD* __restrict__ delta,
-                                   const int* __restrict__ rows, float* __restrict__ out, int D) {
+__global__ void gather_rows_kernel(const float* __restrict__ x, const TD* __restrict__ delta, int parts,
+                                   long long part_stride, const int* __restrict__ rows, float* __restrict__ out,
+                                   int D) {
   const long long src = (long long)rows[blockIdx.x] * D;
   const long long dst = (long long)blockIdx.x * D;
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
     float v = x[src + j];
-    if (HAS_DELTA) v += to_f32(delta[src + j]);
+    if (HAS_DELTA)
+      for (int s = 0; s < parts; ++s) v += to_f32(delta[s * part_stride + src + j]);
     out[dst + j] = v;
   }
 }
 
-extern "C" int lq_gather_rows(const float* x, const void* delta, int delta_dtype, const int* rows,
-                              float* out, int n, int D, hipStream_t stream) {
+extern "C" int lq_gather_rows(const float* x, const void* delta, int delta_dtype, int parts, long long part_stride,
+                              const int* rows, float* out, int n, int D, hipStream_t stream) {
   LQ_REQUIRE(n > 0 && D > 0, "gather_rows: count %d and width %d must be positive", n, D);
   const int threads = D >= 1024 ? 256 : 64;
   if (delta == nullptr)
-    gather_rows_kernel<float, false><<<n, threads, 0, stream>>>(x, nullptr, rows, out, D);
+    gather_rows_kernel<float, false><<<n, threads, 0, stream>>>(x, nullptr, 0, 0, rows, out, D);
   else if (delta_dtype == LQ_F32)
-    gather_rows_kernel<float, true><<<n, threads, 0, stream>>>(x, (const float*)delta, rows, out, D);
+    gather_rows_kernel<float, true><<<n, threads, 0, stream>>>(x, (const float*)delta, parts, part_stride, rows, out, D);
   else if (delta_dtype == LQ_BF16)
-    gather_rows_kernel<bf16_t, true><<<n, threads, 0, stream>>>(x, (const bf16_t*)delta, rows, out, D);
+    gather_rows_kernel<bf16_t, true><<<n, threads, 0, stream>>>(x, (const bf16_t*)delta, parts, part_stride, rows, out, D);
   else
     LQ_REQUIRE(false, "gather_rows: unknown delta dtype %d", delta_dtype);
   LQ_CHECK_LAUNCH("gather_rows");

@@ -5,16 +5,27 @@ int lq_gemm_generic(const void* x, const void* w, void* out, int in_dtype, int o
                     int N, int K, int lda, int ldw, int ldc, hipStream_t stream);
 bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int lda, int ldw);
 int lq_gemm_mfma(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K, int lda,
-                 int ldw, int ldc, int epilogue, hipStream_t stream);
+                 int ldw, int ldc, int epilogue, int splits, long long split_stride, hipStream_t stream);
+int lq_gemm_mfma_splits(int M, int N, int K);
+
+// In how many shares of K lq_linear wants to compute this product (1: whole).  With s > 1 shares the
+// caller passes an output of s pieces, `split_stride` elements apart; their sum is the product, and
+// whoever consumes it adds the pieces in ascending order.
+extern "C" int lq_linear_splits(int in_dtype, int M, int N, int K, int force_generic) {
+  if (force_generic || in_dtype != LQ_BF16 || K % 8 != 0) return 1;
+  return lq_gemm_mfma_splits(M, N, K);
+}
 
 extern "C" int lq_linear(const void* x, const void* w, void* out, int in_dtype, int out_dtype,
-                         int M, int N, int K, int lda, int ldw, int ldc, int force_generic,
-                         hipStream_t stream) {
+                         int M, int N, int K, int lda, int ldw, int ldc, int splits, long long split_stride,
+                         int force_generic, hipStream_t stream) {
   LQ_REQUIRE(M > 0 && N > 0 && K > 0, "linear: sizes M=%d N=%d K=%d must be positive", M, N, K);
   LQ_REQUIRE(lda >= K && ldw >= K && ldc >= N, "linear: a row stride is smaller than its row");
   LQ_REQUIRE(x && w && out, "linear: null pointer");
+  LQ_REQUIRE(splits >= 1 && (splits == 1 || split_stride >= (long long)M * ldc), "linear: bad split arguments");
   if (!force_generic && lq_gemm_mfma_accepts(x, w, in_dtype, K, lda, ldw))
-    return lq_gemm_mfma(x, w, out, out_dtype, M, N, K, lda, ldw, ldc, 0, stream);
+    return lq_gemm_mfma(x, w, out, out_dtype, M, N, K, lda, ldw, ldc, 0, splits, split_stride, stream);
+  LQ_REQUIRE(splits == 1, "linear: only the matrix-core kernels split K");
   return lq_gemm_generic(x, w, out, in_dtype, out_dtype, M, N, K, lda, ldw, ldc, stream);
 }
 
@@ -32,5 +43,5 @@ extern "C" int lq_linear_swiglu(const void* x, const void* w, void* out, int in_
   LQ_REQUIRE(x && w && out, "linear+swiglu: null pointer");
   LQ_REQUIRE(lq_linear_swiglu_supported(in_dtype, N, K) && lq_gemm_mfma_accepts(x, w, in_dtype, K, lda, ldw),
              "linear+swiglu: needs bfloat16, 16-byte aligned rows, K %% 8 == 0 and N %% 16 == 0");
-  return lq_gemm_mfma(x, w, out, out_dtype, M, N, K, lda, ldw, ldc, 1, stream);
+  return lq_gemm_mfma(x, w, out, out_dtype, M, N, K, lda, ldw, ldc, 1, 1, 0, stream);
 }

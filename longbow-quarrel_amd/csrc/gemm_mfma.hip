@@ -295,7 +295,8 @@ template <int KW, int MT, int EPI, typename TO>
 __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16_t* __restrict__ X, int ldx,
                                                                       const bf16_t* __restrict__ W, int ldw,
                                                                       TO* __restrict__ C, int ldc, int M, int N,
-                                                                      int K, int cols_per_block, int ks_per_wave) {
+                                                                      int K, int cols_per_block, int ks_per_wave,
+                                                                      long long split_stride) {
   constexpr int KB = v3_kb(MT);
   constexpr int NBUF = MT == 1 ? 2 : 1;
   constexpr int VALS = MT * 4;  // accumulator values a lane holds per tile
@@ -306,8 +307,11 @@ __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16
   const int col_end = min(N, col_begin + cols_per_block);
   if (col_begin >= N) return;
   const int ntiles = (col_end - col_begin + 15) / 16;
-  const int k_wave = wave * ks_per_wave * 32;  // this wave's slice [k_wave, k_stop)
+  // blockIdx.y: which share of K this block sums (its partial result goes to C + y * split_stride);
+  // within the share, this wave's slice is [k_wave, k_stop)
+  const int k_wave = (blockIdx.y * KW + wave) * ks_per_wave * 32;
   const int k_stop = min(K, k_wave + ks_per_wave * 32);
+  C += blockIdx.y * split_stride;
   const bf16_t* xp[MT];  // k below already holds the lane's g * 8
 #pragma unroll
   for (int m = 0; m < MT; ++m) xp[m] = X + (long long)min(m * 16 + c16, M - 1) * ldx;
@@ -390,11 +394,24 @@ static int lq_compute_units() {
   return n;
 }
 
+// How many blocks should share K for an [M, K] x [N, K]^T product with the balanced kernel (1: no
+// split).  With several row tiles a block wants several column tiles too, so that the x fragments it
+// holds are used more than once; a matrix with few columns gets them by giving each block a wider run
+// of columns and a share of K instead.
+int v3_splits(int M, int N, int K) {
+  if (M <= 16 || M > 64) return 1;
+  if (!(N >= 8 * lq_compute_units() && K >= 512)) return 1;
+  const int tiles_per_block = lq_ceil_div(lq_ceil_div(N, 16), lq_compute_units());
+  int splits = 1;
+  while (splits < 4 && tiles_per_block * splits < 4 && K / (splits * 2) >= 1024) splits *= 2;
+  return splits;
+}
+
 template <int MT, int EPI, typename TO>
 int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc,
-                     hipStream_t stream) {
+                     int splits, long long split_stride, hipStream_t stream) {
   constexpr int KW = v3_kw(MT);
-  const int cus = lq_compute_units();
+  const int cus = lq_compute_units() / splits;
   // equal runs of columns, in units of 16 (8 without the paired epilogue), at most V3_MAXT tiles each
   const int unit = EPI == EPI_SWIGLU ? 16 : 8;
   int blocks = cus;
@@ -405,9 +422,9 @@ int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K,
   }
   const int grid = lq_ceil_div(N, cols);
   const int ksteps = lq_ceil_div(K, 32);
-  const int ks_per_wave = lq_ceil_div(ksteps, KW);
-  gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO><<<grid, KW * 64, 0, stream>>>(
-      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, cols, ks_per_wave);
+  const int ks_per_wave = lq_ceil_div(ksteps, KW * splits);
+  gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO><<<dim3(grid, splits), KW * 64, 0, stream>>>(
+      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, cols, ks_per_wave, split_stride);
   LQ_CHECK_LAUNCH("linear(mfma skinny v3)");
   return 0;
 }
@@ -427,19 +444,27 @@ int pick_skinny(const void* x, const void* w, void* out, int M, int N, int K, in
 
 template <int EPI, typename TO>
 int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
-             hipStream_t stream) {
+             int splits, long long split_stride, hipStream_t stream) {
+  if (splits > 1) {
+    if (EPI != EPI_NONE || splits != v3_splits(M, N, K)) {
+      lq_set_error("linear: %d shares of K are not what this product takes (%d)", splits, v3_splits(M, N, K));
+      return -1;
+    }
+    if (M <= 32) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+    return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+  }
   // wide enough to give every compute unit a run of columns: the balanced kernel; else the simple one
   const bool wide = N >= 8 * lq_compute_units() && K >= 512;
   if (M <= 16) {
-    if (wide) return launch_skinny_v3<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (wide) return launch_skinny_v3<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     return pick_skinny<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
   if (M <= 32) {
-    if (wide) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (wide) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     return pick_skinny<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
   if (M <= 64) {
-    if (wide) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (wide) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     return pick_skinny<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
   // the wider tile reuses each x fragment for twice the columns; it pays once there are enough tiles
@@ -464,23 +489,27 @@ extern "C" int lq_debug_gemm_tiled(const void* x, const void* w, void* out, int 
 }
 
 // Whether the MFMA kernels take this problem (the caller falls back to the generic kernel if not).
+int lq_gemm_mfma_splits(int M, int N, int K) { return v3_splits(M, N, K); }
+
 bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int lda, int ldw) {
   return in_dtype == LQ_BF16 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 &&
          ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
 }
 
 int lq_gemm_mfma(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K, int lda,
-                 int ldw, int ldc, int epilogue, hipStream_t stream) {
+                 int ldw, int ldc, int epilogue, int splits, long long split_stride, hipStream_t stream) {
   if (epilogue == EPI_NONE) {
-    if (out_dtype == LQ_F32) return dispatch<EPI_NONE, float>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-    if (out_dtype == LQ_BF16) return dispatch<EPI_NONE, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (out_dtype == LQ_F32)
+      return dispatch<EPI_NONE, float>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+    if (out_dtype == LQ_BF16)
+      return dispatch<EPI_NONE, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
   } else if (epilogue == EPI_SWIGLU) {
     if (N % 16 != 0) {
       lq_set_error("linear+swiglu: %d interleaved rows are not a multiple of 16", N);
       return -1;
     }
-    if (out_dtype == LQ_F32) return dispatch<EPI_SWIGLU, float>(x, w, out, M, N, K, lda, ldw, ldc, stream);
-    if (out_dtype == LQ_BF16) return dispatch<EPI_SWIGLU, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+    if (out_dtype == LQ_F32) return dispatch<EPI_SWIGLU, float>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    if (out_dtype == LQ_BF16) return dispatch<EPI_SWIGLU, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
   }
   lq_set_error("linear: unknown out dtype %d or epilogue %d", out_dtype, epilogue);
   return -1;

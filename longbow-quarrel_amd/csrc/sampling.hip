@@ -125,18 +125,44 @@ __global__ __launch_bounds__(RECENT) void penalty_kernel(float* __restrict__ log
 }
 
 // ------------------------------------------------------------------ greedy
-__global__ __launch_bounds__(THREADS) void argmax_kernel(const float* __restrict__ logits, int ld, int V,
-                                                         const int* __restrict__ seq_slot, int* __restrict__ out,
-                                                         int* __restrict__ recent, int* __restrict__ recent_n) {
-  __shared__ unsigned long long sm[THREADS / 64];
-  const int row = blockIdx.x;
+// Two stages so that a few rows still use many compute units: ARGMAX_PARTS blocks a row reduce a
+// slice of the vocabulary each to its best key, one block a row reduces those.  Keys order by logit,
+// then by lower index, so the result is the first maximal index whatever the slicing.
+constexpr int ARGMAX_PARTS = 32;
+
+__global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ logits, int ld, int V,
+                                                          unsigned long long* __restrict__ part) {
+  __shared__ unsigned long long sm[4];
+  const int row = blockIdx.y, slice = blockIdx.x;
   const float* lr = logits + (long long)row * ld;
+  const int per = (V + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+  const int i1 = min(V, (slice + 1) * per);
   unsigned long long best = 0ull;
-  for (int i = threadIdx.x; i < V; i += THREADS) {
+  for (int i = slice * per + threadIdx.x; i < i1; i += 256) {
     const unsigned long long k = key_of(lr[i], i);
     best = k > best ? k : best;
   }
-  best = block_max_u64(best, sm);
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned long long o = shfl_xor_u64(best, off);
+    best = o > best ? o : best;
+  }
+  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) best = sm[w] > best ? sm[w] : best;
+    part[(long long)row * ARGMAX_PARTS + slice] = best;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const unsigned long long* __restrict__ part,
+                                                          const int* __restrict__ seq_slot, int* __restrict__ out,
+                                                          int* __restrict__ recent, int* __restrict__ recent_n) {
+  const int row = blockIdx.x;
+  unsigned long long best = threadIdx.x < ARGMAX_PARTS ? part[(long long)row * ARGMAX_PARTS + threadIdx.x] : 0ull;
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned long long o = shfl_xor_u64(best, off);
+    best = o > best ? o : best;
+  }
   if (threadIdx.x == 0) {
     const int tok = (int)(0xffffffffu - (unsigned)(best & 0xffffffffull));
     out[row] = tok;
@@ -360,16 +386,6 @@ __global__ void advance_kernel(int* row_pos, int* seq_start, int* seq_len, int b
   }
 }
 
-__global__ void record_kernel(const int* tokens, int* history, int batch, const int* step_index, int max_steps) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  const int s = *step_index;
-  if (i < batch && s < max_steps) history[(long long)s * batch + i] = tokens[i];
-}
-
-__global__ void bump_kernel(int* step_index) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) *step_index += 1;
-}
-
 }  // namespace
 
 extern "C" int lq_apply_penalty(float* logits, int ld, int rows, int V, const int* seq_slot, const int* recent,
@@ -381,11 +397,15 @@ extern "C" int lq_apply_penalty(float* logits, int ld, int rows, int V, const in
   return 0;
 }
 
+// `scratch`: rows * 32 64-bit words the two stages pass their partial results through
 extern "C" int lq_argmax(const float* logits, int ld, int rows, int V, const int* seq_slot, int* out, int* recent,
-                         int* recent_n, hipStream_t stream) {
+                         int* recent_n, unsigned long long* scratch, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && V > 0 && ld >= V, "argmax: bad sizes");
+  LQ_REQUIRE(rows <= 65535, "argmax: %d rows are too many for one launch", rows);
+  LQ_REQUIRE(scratch != nullptr, "argmax: scratch of rows * %d 64-bit words is needed", ARGMAX_PARTS);
   LQ_REQUIRE(recent == nullptr || (recent_n != nullptr && seq_slot != nullptr), "argmax: ring without its counters");
-  argmax_kernel<<<rows, THREADS, 0, stream>>>(logits, ld, V, seq_slot, out, recent, recent_n);
+  argmax_part_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, stream>>>(logits, ld, V, scratch);
+  argmax_final_kernel<<<rows, 64, 0, stream>>>(scratch, seq_slot, out, recent, recent_n);
   LQ_CHECK_LAUNCH("argmax");
   return 0;
 }
@@ -421,15 +441,5 @@ extern "C" int lq_advance(int* row_pos, int* seq_start, int* seq_len, int batch,
   LQ_REQUIRE(batch > 0, "advance: batch %d must be positive", batch);
   advance_kernel<<<lq_ceil_div(batch, 256), 256, 0, stream>>>(row_pos, seq_start, seq_len, batch);
   LQ_CHECK_LAUNCH("advance");
-  return 0;
-}
-
-// history[*step_index][:] = tokens; then *step_index += 1
-extern "C" int lq_record(const int* tokens, int* history, int batch, int* step_index, int max_steps,
-                         hipStream_t stream) {
-  LQ_REQUIRE(batch > 0 && max_steps > 0, "record: bad sizes");
-  record_kernel<<<lq_ceil_div(batch, 256), 256, 0, stream>>>(tokens, history, batch, step_index, max_steps);
-  bump_kernel<<<1, 64, 0, stream>>>(step_index);
-  LQ_CHECK_LAUNCH("record");
   return 0;
 }

@@ -121,10 +121,21 @@ class HipKernels:
         self._check(self.lib.lq_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(out),
                                       c_int(rows), c_int(width), self.stream))
 
+    @staticmethod
+    def _pieces(delta: Optional[torch.Tensor], like: torch.Tensor, what: str):
+        """A delta is shaped like x, or holds several pieces [pieces, rows, width] whose sum is meant
+        (`linear_pieces`).  -> (pieces, elements between pieces)"""
+        if delta is None:
+            return 0, 0
+        if not delta.is_contiguous() or tuple(delta.shape[-2:]) != tuple(like.shape) or delta.dim() not in (2, 3):
+            raise KernelLibraryError(f"{what}: delta must be dense and shaped like x, or a stack of such pieces")
+        return (delta.shape[0], like.numel()) if delta.dim() == 3 else (1, 0)
+
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
                 delta: Optional[torch.Tensor] = None) -> None:
         """(x += delta;) out = x / sqrt(mean(x^2) + eps) * weight, row by row; x is float32."""
         self._dev(x, weight, out, delta)
+        pieces, stride = self._pieces(delta, x, "rmsnorm")
         rows, width = x.shape
         if x.dtype != torch.float32 or not x.is_contiguous():
             raise KernelLibraryError("rmsnorm: x must be dense float32")
@@ -132,18 +143,20 @@ class HipKernels:
             raise KernelLibraryError(f"rmsnorm: weight must be float32 of {width} entries")
         if tuple(out.shape) != (rows, width) or not out.is_contiguous():
             raise KernelLibraryError("rmsnorm: out must be dense and shaped like x")
-        if delta is not None and (tuple(delta.shape) != (rows, width) or not delta.is_contiguous()):
-            raise KernelLibraryError("rmsnorm: delta must be dense and shaped like x")
         self._check(self.lib.lq_rmsnorm(_ptr(x), _ptr(delta), c_int(_code(delta) if delta is not None else 0),
+                                        c_int(pieces), c_longlong(stride),
                                         _ptr(weight), c_float(eps), _ptr(out), c_int(_code(out)),
                                         c_int(rows), c_int(width), self.stream))
 
     def add(self, x: torch.Tensor, delta: torch.Tensor) -> None:
         """x += delta (x float32)."""
         self._dev(x, delta)
-        if x.dtype != torch.float32 or x.shape != delta.shape or not x.is_contiguous() or not delta.is_contiguous():
-            raise KernelLibraryError("add: x must be dense float32 and delta dense of the same shape")
-        self._check(self.lib.lq_add(_ptr(x), _ptr(delta), c_int(_code(delta)), c_longlong(x.numel()), self.stream))
+        if x.dtype != torch.float32 or not x.is_contiguous():
+            raise KernelLibraryError("add: x must be dense float32")
+        pieces, _ = self._pieces(delta, x, "add")
+        for piece in (delta if pieces > 1 or delta.dim() == 3 else (delta,)):
+            self._check(self.lib.lq_add(_ptr(x), _ptr(piece), c_int(_code(piece)), c_longlong(x.numel()),
+                                        self.stream))
 
     def cast(self, src: torch.Tensor, out: torch.Tensor) -> None:
         self._dev(src, out)
@@ -152,21 +165,38 @@ class HipKernels:
         self._check(self.lib.lq_cast(_ptr(src), c_int(_code(src)), _ptr(out), c_int(_code(out)),
                                      c_longlong(src.numel()), self.stream))
 
+    def linear_pieces(self, dtype: torch.dtype, m: int, n: int, k: int) -> int:
+        """In how many pieces `linear` would like to leave this product (1: whole).  A caller whose
+        consumer adds pieces (`rmsnorm`, `add`, `gather_rows` with a stacked delta) may pass an output
+        [pieces, M, N]; the kernel then splits K over more blocks and each piece is a partial sum."""
+        if dtype not in _DTYPE_CODE:
+            return 1
+        return int(self.lib.lq_linear_splits(c_int(_DTYPE_CODE[dtype]), c_int(m), c_int(n), c_int(k),
+                                             c_int(1 if self.force_generic else 0)))
+
     def linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
-        """out[M, N] = x[M, K] . w[N, K]^T with 32-bit accumulation."""
+        """out[M, N] = x[M, K] . w[N, K]^T with 32-bit accumulation; or out[pieces, M, N] with
+        `linear_pieces` pieces that sum to it."""
         self._dev(x, w, out)
-        if x.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+        if x.dim() != 2 or w.dim() != 2 or out.dim() not in (2, 3):
             raise KernelLibraryError("linear: 2-D tensors are needed")
         m, k = x.shape
         n = w.shape[0]
-        if w.shape[1] != k or tuple(out.shape) != (m, n):
+        if w.shape[1] != k or tuple(out.shape[-2:]) != (m, n):
             raise KernelLibraryError(
                 f"linear: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
         if x.dtype != w.dtype:
             raise KernelLibraryError(f"linear: x is {x.dtype} but w is {w.dtype}")
+        pieces, stride = 1, 0
+        if out.dim() == 3:
+            pieces, stride = out.shape[0], m * n
+            if not out.is_contiguous() or pieces != self.linear_pieces(x.dtype, m, n, k):
+                raise KernelLibraryError(f"linear: {pieces} pieces asked, linear_pieces says "
+                                         f"{self.linear_pieces(x.dtype, m, n, k)}")
+        ldc = self._rows2d(out[0], "out") if out.dim() == 3 else self._rows2d(out, "out")
         self._check(self.lib.lq_linear(_ptr(x), _ptr(w), _ptr(out), c_int(_code(x)), c_int(_code(out)),
                                        c_int(m), c_int(n), c_int(k), c_int(self._rows2d(x, "x")),
-                                       c_int(self._rows2d(w, "w")), c_int(self._rows2d(out, "out")),
+                                       c_int(self._rows2d(w, "w")), c_int(ldc), c_int(pieces), c_longlong(stride),
                                        c_int(1 if self.force_generic else 0), self.stream))
 
     def linear_swiglu_supported(self, dtype: torch.dtype, rows_out: int, k: int) -> bool:
@@ -214,13 +244,13 @@ class HipKernels:
         self._dev(x, rows, out, delta)
         n, width = out.shape
         self._i32(rows, "gather rows", n)
+        pieces, stride = self._pieces(delta, x, "gather_rows")
         if x.dtype != torch.float32 or out.dtype != torch.float32 or x.shape[1] != width:
             raise KernelLibraryError("gather_rows: float32 tensors of one width are needed")
         if not x.is_contiguous() or not out.is_contiguous():
             raise KernelLibraryError("gather_rows: dense tensors are needed")
-        if delta is not None and (delta.shape != x.shape or not delta.is_contiguous()):
-            raise KernelLibraryError("gather_rows: delta must be dense and shaped like x")
         self._check(self.lib.lq_gather_rows(_ptr(x), _ptr(delta), c_int(_code(delta) if delta is not None else 0),
+                                            c_int(pieces), c_longlong(stride),
                                             _ptr(rows), _ptr(out), c_int(n), c_int(width), self.stream))
 
     def rope_store(self, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
@@ -367,19 +397,23 @@ class HipKernels:
                                               c_int(vocab), _ptr(seq_slot), _ptr(recent), _ptr(recent_n),
                                               c_float(penalty), self.stream))
 
-    def argmax(self, logits: torch.Tensor, out: torch.Tensor, seq_slot: Optional[torch.Tensor] = None,
-               recent: Optional[torch.Tensor] = None, recent_n: Optional[torch.Tensor] = None) -> None:
-        """out[r] = first maximal index of logits[r]; the token is pushed into the ring if one is given."""
-        self._dev(logits, out, seq_slot, recent, recent_n)
+    def argmax(self, logits: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor,
+               seq_slot: Optional[torch.Tensor] = None, recent: Optional[torch.Tensor] = None,
+               recent_n: Optional[torch.Tensor] = None) -> None:
+        """out[r] = first maximal index of logits[r]; the token is pushed into the ring if one is given.
+        `scratch`: int64 with at least 32 entries a row."""
+        self._dev(logits, out, scratch, seq_slot, recent, recent_n)
         rows, vocab = logits.shape
         self._i32(out, "argmax out", rows)
         if logits.dtype != torch.float32:
             raise KernelLibraryError("argmax: logits must be float32")
+        if scratch.dtype != torch.int64 or not scratch.is_contiguous() or scratch.numel() < 32 * rows:
+            raise KernelLibraryError(f"argmax: scratch must be dense int64 with at least {32 * rows} entries")
         if recent is not None:
             self._i32(seq_slot, "seq_slot", rows)
         self._check(self.lib.lq_argmax(_ptr(logits), c_int(self._rows2d(logits, "logits")), c_int(rows),
                                        c_int(vocab), _ptr(seq_slot), _ptr(out), _ptr(recent), _ptr(recent_n),
-                                       self.stream))
+                                       _ptr(scratch), self.stream))
 
     def sample(self, logits: torch.Tensor, out: torch.Tensor, seq_slot: torch.Tensor, temperature: float,
                top_k: int, top_p: float, rng_key: torch.Tensor, rng_ctr: torch.Tensor,
@@ -407,16 +441,6 @@ class HipKernels:
         for t in (row_pos, seq_start, seq_len):
             self._i32(t, "advance", batch)
         self._check(self.lib.lq_advance(_ptr(row_pos), _ptr(seq_start), _ptr(seq_len), c_int(batch), self.stream))
-
-    def record(self, tokens: torch.Tensor, history: torch.Tensor, step_index: torch.Tensor, batch: int) -> None:
-        """history[step_index] = tokens; step_index += 1 (nothing is written past the last row)."""
-        self._dev(tokens, history, step_index)
-        self._i32(tokens, "record tokens", batch)
-        if history.dtype != torch.int32 or history.dim() != 2 or history.shape[1] != batch or not history.is_contiguous():
-            raise KernelLibraryError("record: history must be dense int32 [steps, batch]")
-        self._i32(step_index, "step_index", 1)
-        self._check(self.lib.lq_record(_ptr(tokens), _ptr(history), c_int(batch), _ptr(step_index),
-                                       c_int(history.shape[0]), self.stream))
 
     # ------------------------------------------------------------------ HIP graphs
     def graph_begin(self) -> None:

@@ -18,7 +18,7 @@ from typing import Dict, List, Mapping, Optional
 import torch
 
 from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mixer, PartSpec,
-                   StepContext, TensorSpec, build_part, project)
+                   StepContext, TensorSpec, build_part, project, project_delta)
 
 
 @MIXERS.register("gqa_attention")
@@ -99,6 +99,4 @@ class GQAttention(Mixer):
             kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
                          ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
                          self.scale, self.window, decode=ctx.decode, max_len=ctx.max_len, workspace=scratch)
-        out = ctx.ws.alloc((rows, self.width), torch.float32)
-        project(kn, ctx, att, self.w_o, out)
-        return out
+        return project_delta(kn, ctx, att, self.w_o)

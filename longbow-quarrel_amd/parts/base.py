@@ -286,6 +286,16 @@ def build_part(registry: Registry, spec: PartSpec, **extra):
     return cls(**dict(spec.params), **extra)
 
 
+def project_delta(kn, ctx: StepContext, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x . w^T as a float32 delta for the residual stream: [rows, N], or [pieces, rows, N] where the
+    kernels prefer to leave partial sums (whoever adds the delta adds the pieces, in order)."""
+    rows, n = x.shape[0], w.shape[0]
+    pieces = kn.linear_pieces(x.dtype, rows, n, x.shape[1]) if w.dtype == x.dtype else 1
+    out = ctx.ws.alloc((pieces, rows, n) if pieces > 1 else (rows, n), torch.float32)
+    project(kn, ctx, x, w, out)
+    return out
+
+
 def project(kn, ctx: StepContext, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     """out = x . w^T.  A weight stored in 32-bit is used in 32-bit: bfloat16
     activations are widened for it rather than the weight narrowed."""

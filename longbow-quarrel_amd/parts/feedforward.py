@@ -8,7 +8,7 @@ from typing import Dict, List, Mapping, Optional
 
 import torch
 
-from .base import FEED_FORWARDS, BuildEnv, FeedForward, StepContext, TensorSpec, project
+from .base import FEED_FORWARDS, BuildEnv, FeedForward, StepContext, TensorSpec, project, project_delta
 
 
 @FEED_FORWARDS.register("swiglu")
@@ -56,6 +56,4 @@ class SwiGLU(FeedForward):
             gu = ctx.ws.alloc((rows, 2 * self.inner), torch.float32)
             project(kn, ctx, h, self.w_gate_up, gu)
             kn.swiglu(gu, act)
-        out = ctx.ws.alloc((rows, self.width), torch.float32)
-        project(kn, ctx, act, self.w_down, out)
-        return out
+        return project_delta(kn, ctx, act, self.w_down)

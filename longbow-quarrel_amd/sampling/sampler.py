@@ -27,7 +27,7 @@ class Sampler:
         if p.repetition_penalty > 1.0:
             kn.apply_penalty(logits, seq_slot, st.recent, st.recent_n, p.repetition_penalty)
         if p.greedy:
-            kn.argmax(logits, out, seq_slot, st.recent, st.recent_n)
+            kn.argmax(logits, out, st.argmax_scratch, seq_slot, st.recent, st.recent_n)
         else:
             kn.sample(logits, out, seq_slot, p.temperature, p.top_k, p.top_p, st.rng_key, st.rng_ctr,
                       st.recent, st.recent_n)

@@ -29,6 +29,8 @@ class SamplerState:
         self.rng_ctr = torch.zeros(max_slots, dtype=torch.int64, device=device)
         self.recent = torch.full((max_slots, RECENT), -1, dtype=torch.int32, device=device)
         self.recent_n = torch.zeros(max_slots, dtype=torch.int32, device=device)
+        # what the two stages of the arg-max kernel pass between them: 32 words for each row of a batch
+        self.argmax_scratch = torch.zeros(32 * max_slots, dtype=torch.int64, device=device)
 
     def start(self, slot: int, key: int, history: Sequence[int]) -> None:
         """A sequence starts in `slot`: generator at draw 0, ring holding the end of its prompt."""

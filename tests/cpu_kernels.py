@@ -26,14 +26,22 @@ class CpuKernels:
     def embed(self, table, tokens, out):
         out.copy_(table[tokens[: out.shape[0]].long()].float())
 
+    @staticmethod
+    def _whole(delta, like):
+        d = delta.float()
+        return d.sum(0) if d.dim() == like.dim() + 1 else d
+
+    def linear_pieces(self, dtype, m, n, k):
+        return 1
+
     def rmsnorm(self, x, weight, eps, out, delta=None):
         if delta is not None:
-            x += delta.float()
+            x += self._whole(delta, x)
         ms = (x * x).sum(-1, keepdim=True) / x.shape[-1]
         out.copy_((x / torch.sqrt(ms + eps) * weight).to(out.dtype))
 
     def add(self, x, delta):
-        x += delta.float()
+        x += self._whole(delta, x)
 
     def cast(self, src, out):
         out.copy_(src.to(out.dtype))
@@ -52,7 +60,7 @@ class CpuKernels:
         idx = rows[: out.shape[0]].long()
         v = x[idx]
         if delta is not None:
-            v = v + delta[idx].float()
+            v = v + self._whole(delta, x)[idx]
         out.copy_(v)
 
     @staticmethod

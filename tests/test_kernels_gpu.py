@@ -122,6 +122,42 @@ def test_linear_bfloat16_matrix_cores(kn, out_dtype, m, n, k):
     assert rel_err(out, want) < (1e-5 if out_dtype == torch.float32 else 5e-3)
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 4096, 4096), (17, 4096, 14336), (40, 2560, 2056), (33, 6144, 4096)])
+def test_linear_in_pieces_and_their_consumers(kn, m, n, k):
+    """Few columns and several row tiles: K is shared out over blocks and the product comes as
+    pieces; the norm, the add and the row gather that take such a delta add the pieces up."""
+    pieces = kn.linear_pieces(torch.bfloat16, m, n, k)
+    assert pieces > 1
+    assert kn.linear_pieces(torch.bfloat16, 8, n, k) == 1 and kn.linear_pieces(torch.float32, m, n, k) == 1
+    x, w = rnd((m, k), 40, torch.bfloat16), rnd((n, k), 41, torch.bfloat16)
+    out = torch.full((pieces, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    kn.linear(x, w, out)
+    want = x.double().cpu() @ w.double().cpu().t()
+    assert rel_err(out.double().sum(0), want) < 1e-5
+    whole = torch.empty((m, n), dtype=torch.float32, device=DEV)
+    kn.linear(x, w, whole)
+    assert rel_err(whole, want) < 1e-5
+    from longbow_quarrel_amd.kernels.hip import KernelLibraryError
+
+    with pytest.raises(KernelLibraryError):
+        kn.linear(x, w, torch.empty((pieces + 1, m, n), dtype=torch.float32, device=DEV))
+
+    res = rnd((m, n), 42)
+    summed = res.double().cpu() + want
+    r1, normed = res.clone(), torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    nw = rnd((n,), 43)
+    kn.rmsnorm(r1, nw, 1e-5, normed, delta=out)
+    assert rel_err(r1, summed) < 1e-6
+    assert rel_err(normed, plain.rms_norm(summed, nw.cpu(), 1e-5)) < 5e-3
+    r2 = res.clone()
+    kn.add(r2, out)
+    assert rel_err(r2, summed) < 1e-6
+    rows = i32([m - 1, 0, 5])
+    picked = torch.empty((3, n), dtype=torch.float32, device=DEV)
+    kn.gather_rows(res, rows, picked, delta=out)
+    assert rel_err(picked, summed[rows.long().cpu()]) < 1e-6
+
+
 def test_linear_bfloat16_odd_k_takes_the_generic_kernel(kn):
     x, w = rnd((9, 77), 14, torch.bfloat16), rnd((33, 77), 15, torch.bfloat16)
     out = torch.empty((9, 33), dtype=torch.float32, device=DEV)

@@ -57,7 +57,7 @@ def run(kn, logits, params, slots=None, state=None, history=None):
     if params.repetition_penalty > 1:
         kn.apply_penalty(lg, seq_slot, state.recent, state.recent_n, params.repetition_penalty)
     if params.greedy:
-        kn.argmax(lg, out, seq_slot, state.recent, state.recent_n)
+        kn.argmax(lg, out, state.argmax_scratch, seq_slot, state.recent, state.recent_n)
     else:
         kn.sample(lg, out, seq_slot, params.temperature, params.top_k, params.top_p, state.rng_key, state.rng_ctr,
                   state.recent, state.recent_n, kept, mass)
@@ -70,6 +70,12 @@ def test_reference_vectors(kn):
     assert tok == [1]
     tok, *_ = run(kn, torch.tensor([[2.0, 7.0, 7.0, 7.0]]), SamplingParams())
     assert tok == [1]  # first maximal index
+    wide = torch.zeros((3, 128256))
+    wide[0, [99999, 500, 128255]] = 4.0   # equal maxima in different slices of the vocabulary
+    wide[1, 128255] = 1.0
+    wide[2] = -1.0
+    tok, *_ = run(kn, wide, SamplingParams())
+    assert tok == [500, 128255, 0]
     for seed in range(30):
         h = [[0]] 
         tok, kept, *_ = run(kn, torch.tensor([[2.0, 10.0, 5.0, 1.0]]), SamplingParams(temperature=1.0, top_k=1, seed=seed), history=h)
