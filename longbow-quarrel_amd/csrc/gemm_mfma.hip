@@ -8,10 +8,13 @@
 //   v_mfma_f32_16x16x32_bf16: lane l gives A[row l%16][k (l/16)*8 .. +8] and
 //     B[col l%16][same k]; it receives D[(l/16)*4 + e][l%16], e < 4.
 //
-// Two kernels:
+// Kernels:
+//  * tiled, pipelined: 4 or 8 waves compute a 128 x 256 or 256 x 256 tile; operand slabs go from
+//    memory straight into a ring of LDS stages (no registers in between).  For many rows (prefill)
+//    and K a multiple of 32.
 //  * tiled: a block of 4 waves (2 x 2) computes a (2*WM*32) x (2*WN*32) tile, operands staged
 //    through padded LDS in steps of 64 k, next step prefetched into registers while the current one
-//    is multiplied.  For many rows (prefill).
+//    is multiplied.  Takes any K that is a multiple of 8, and the small cases.
 //  * skinny: at most 16 rows (decode).  A block owns 16 output columns; its KW waves split K,
 //    stream their slice of the 16 weight rows straight from memory into MFMA operands (every
 //    weight byte is read once, 16 bytes a lane), and add their partial tiles through LDS in
@@ -55,6 +58,30 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
 enum { EPI_NONE = 0, EPI_SWIGLU = 1 };
 
 __device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
+// A wave's WM x WN accumulators of 32 x 32 go to C (rows from row0, columns from col0).
+template <int WM, int WN, int EPI, typename TO>
+__device__ inline void tile_epilogue(f32x16 (&acc)[WM][WN], TO* __restrict__ C, int ldc, int M, int N, int row0,
+                                     int col0, int lane) {
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int col = col0 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = row0 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (EPI == EPI_SWIGLU) {
+          // gate column c (c % 16 < 8) and its up column c + 8 sit 8 lanes apart
+          const float up = __shfl(acc[i][j][e], lane + 8, 64);
+          if ((col & 15) < 8 && row < M && col + 8 < N)
+            store_out<TO>(C + (long long)row * ldc + ((col >> 4) << 3) + (col & 7), silu_mul(acc[i][j][e], up));
+        } else {
+          if (row < M && col < N) store_out<TO>(C + (long long)row * ldc + col, acc[i][j][e]);
+        }
+      }
+    }
+}
 
 // ------------------------------------------------------------------ tiled
 constexpr int TBK = 64;           // k per stage
@@ -148,24 +175,7 @@ __global__ __launch_bounds__(256, (WM * WN <= 8 ? 2 : 1)) void gemm_bf16_tiled_k
     }
   }
 
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      const int col = n0 + wn * WN * 32 + j * 32 + (lane & 31);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm * WM * 32 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (EPI == EPI_SWIGLU) {
-          // gate column c (c % 16 < 8) and its up column c + 8 sit 8 lanes apart
-          const float up = __shfl(acc[i][j][e], lane + 8, 64);
-          if ((col & 15) < 8 && row < M && col + 8 < N)
-            store_out<TO>(C + (long long)row * ldc + ((col >> 4) << 3) + (col & 7), silu_mul(acc[i][j][e], up));
-        } else {
-          if (row < M && col < N) store_out<TO>(C + (long long)row * ldc + col, acc[i][j][e]);
-        }
-      }
-    }
+  tile_epilogue<WM, WN, EPI, TO>(acc, C, ldc, M, N, m0 + wm * WM * 32, n0 + wn * WN * 32, lane);
 }
 
 template <int WM, int WN, int EPI, typename TO>
@@ -190,6 +200,177 @@ int launch_tiled(const void* A, const void* W, void* C, int M, int N, int K, int
   kernel<<<(int)blocks, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, (TO*)C, ldc,
                                               M, N, K, tiles_m, tiles_n);
   LQ_CHECK_LAUNCH("linear(mfma tiled)");
+  return 0;
+}
+
+// ------------------------------------------------------------------ tiled, pipelined
+// What bounds a large product here is the traffic from L2 into the compute units, so this kernel
+// makes the block tile large (GM x GN waves, each WM x WN accumulators of 32 x 32) and moves operand
+// slabs of BK k from memory straight into LDS (global_load_lds_dwordx4: no registers, no LDS store
+// instructions) into a ring of STAGES stages, STAGES - 1 slabs ahead of the one being multiplied, with
+// one barrier a slab.  LDS rows are BK * 2 bytes, unpadded; the 16-byte chunk c of row r sits at chunk
+// position c ^ swizzle(r), which keeps a fragment read (16 consecutive rows, one chunk) on 16
+// different bank groups.  Fragment reads run two 16-k steps ahead of the products.
+// blockIdx.y shares K: each share writes its partial product to C + y * split_stride.
+// Needs K % (BK * shares) == 0.
+#define LQ_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define LQ_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters at their maxima)
+#define LQ_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+
+template <int GM, int GN, int WM, int WN, int BK, int STAGES>
+struct PipeShape {
+  static constexpr int NW = GM * GN;                        // waves
+  static constexpr int BM = GM * WM * 32, BN = GN * WN * 32;
+  static constexpr int ROW_BYTES = BK * 2;
+  static constexpr int CPR = BK / 8;                        // 16-byte chunks a row
+  static constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;     // a wave's transfer is 64 lanes x 16 bytes
+  static constexpr int A_DMA = BM / ROWS_PER_DMA / NW, W_DMA = BN / ROWS_PER_DMA / NW;
+  static constexpr int A_BYTES = BM * ROW_BYTES, STAGE_BYTES = (BM + BN) * ROW_BYTES;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int KK = BK / 16;                        // 16-k steps a slab
+  static_assert(BM % (ROWS_PER_DMA * NW) == 0 && BN % (ROWS_PER_DMA * NW) == 0, "transfers must deal out evenly");
+  static_assert((A_DMA + W_DMA) * (STAGES - 1) < 64, "vmcnt has 6 bits");
+  // chunk position of chunk c in row r: rows that share a 256-byte bank row get different positions
+  __device__ static int swizzle(int row) { return (row / (256 / ROW_BYTES)) & (CPR - 1); }
+};
+
+template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO>
+__global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
+    const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw, TO* __restrict__ C, int ldc, int M,
+    int N, int K, int tiles_m, int tiles_n, int k_share, long long split_stride) {
+  using S = PipeShape<GM, GN, WM, WN, BK, STAGES>;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char plds[];
+
+  const int total = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  if (total % 8 == 0) pid = (pid % 8) * (total / 8) + pid / 8;  // one XCD walks a contiguous run of tiles
+  const int tm = pid % tiles_m, tn = pid / tiles_m;
+  const int m0 = tm * S::BM, n0 = tn * S::BN;
+  const int k_begin = blockIdx.y * k_share;
+  C += blockIdx.y * split_stride;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / GN, wn = wave % GN;
+
+  // where this lane's 16 bytes of each transfer come from: transfer j of the wave fills the LDS
+  // chunks [(NW j + wave) * 64, + 64); chunk p is row p / CPR, position p % CPR
+  const bf16_t* pa[S::A_DMA];
+  const bf16_t* pw[S::W_DMA];
+#pragma unroll
+  for (int j = 0; j < S::A_DMA; ++j) {
+    const int p = (j * S::NW + wave) * 64 + lane, row = p / S::CPR, c = (p % S::CPR) ^ S::swizzle(row);
+    pa[j] = A + (long long)min(m0 + row, M - 1) * lda + k_begin + c * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < S::W_DMA; ++j) {
+    const int p = (j * S::NW + wave) * 64 + lane, row = p / S::CPR, c = (p % S::CPR) ^ S::swizzle(row);
+    pw[j] = W + (long long)min(n0 + row, N - 1) * ldw + k_begin + c * 8;
+  }
+  auto dma = [&](int stage, int k0) {
+    unsigned char* base = plds + stage * S::STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < S::A_DMA; ++j)
+      __builtin_amdgcn_global_load_lds(LQ_GLOBAL_PTR(pa[j] + k0), LQ_LDS_PTR(base + (j * S::NW + wave) * 1024), 16, 0,
+                                       0);
+#pragma unroll
+    for (int j = 0; j < S::W_DMA; ++j)
+      __builtin_amdgcn_global_load_lds(LQ_GLOBAL_PTR(pw[j] + k0),
+                                       LQ_LDS_PTR(base + S::A_BYTES + (j * S::NW + wave) * 1024), 16, 0, 0);
+  };
+
+  // fragment addresses within a 32-row group: row lane % 32, chunk 2 kk + lane / 32, swizzled
+  int frag[S::KK];
+#pragma unroll
+  for (int kk = 0; kk < S::KK; ++kk)
+    frag[kk] = (lane & 31) * S::ROW_BYTES + ((2 * kk + (lane >> 5)) ^ S::swizzle(lane & 31)) * 16;
+  const unsigned char* a_base = plds + wm * WM * 32 * S::ROW_BYTES;
+  const unsigned char* w_base = plds + S::A_BYTES + wn * WN * 32 * S::ROW_BYTES;
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int slabs = k_share / BK;
+#pragma unroll
+  for (int q = 0; q < STAGES - 1; ++q)
+    if (q < slabs) dma(q, q * BK);
+
+  auto step = [&](int stage, int t) {
+    // this wave's transfers of slab t have landed (those of the slabs behind it may still fly) ...
+    const int behind = min(STAGES - 2, slabs - 1 - t);
+    if (STAGES >= 4 && behind == 2)
+      LQ_WAIT_VMCNT(2 * (S::A_DMA + S::W_DMA));
+    else if (STAGES >= 3 && behind == 1)
+      LQ_WAIT_VMCNT(S::A_DMA + S::W_DMA);
+    else
+      LQ_WAIT_VMCNT(0);
+    // ... and so have everyone's; and everyone is done reading slab t - 1, whose stage is filled next
+    asm volatile("s_barrier" ::: "memory");
+    if (t + STAGES - 1 < slabs) dma((stage + STAGES - 1) % STAGES, (t + STAGES - 1) * BK);
+    const unsigned char* as = a_base + stage * S::STAGE_BYTES;
+    const unsigned char* ws = w_base + stage * S::STAGE_BYTES;
+    bf16x8 a[2][WM], b[2][WN];
+    auto read = [&](int kk) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        a[kk & 1][i] = as_bf16x8(*(const u32x4*)(as + i * 32 * S::ROW_BYTES + frag[kk]));
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        b[kk & 1][j] = as_bf16x8(*(const u32x4*)(ws + j * 32 * S::ROW_BYTES + frag[kk]));
+    };
+    read(0);
+    read(1);
+#pragma unroll
+    for (int kk = 0; kk < S::KK; ++kk) {
+      __builtin_amdgcn_sched_barrier(0);  // reads stay ahead of the products they do not feed
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk & 1][i], b[kk & 1][j], acc[i][j], 0, 0, 0);
+      if (kk + 2 < S::KK) read(kk + 2);
+    }
+  };
+  static_assert(STAGES >= 2 && STAGES <= 4, "the wait above knows 2 to 4 stages");
+  for (int t = 0; t < slabs; t += STAGES) {
+#pragma unroll
+    for (int q = 0; q < STAGES; ++q)
+      if (t + q < slabs) step(q, t + q);
+  }
+  tile_epilogue<WM, WN, EPI, TO>(acc, C, ldc, M, N, m0 + wm * WM * 32, n0 + wn * WN * 32, lane);
+}
+
+template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO>
+int launch_pipelined(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
+                     int splits, long long split_stride, hipStream_t stream) {
+  using S = PipeShape<GM, GN, WM, WN, BK, STAGES>;
+  const int tiles_m = lq_ceil_div(M, S::BM), tiles_n = lq_ceil_div(N, S::BN);
+  auto kernel = gemm_bf16_pipelined_kernel<GM, GN, WM, WN, BK, STAGES, EPI, TO>;
+  static bool configured = false;
+  if (!configured && S::LDS_BYTES > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       S::LDS_BYTES);
+    if (e != hipSuccess) {
+      lq_set_error("linear: cannot reserve %d bytes of LDS: %s", S::LDS_BYTES, hipGetErrorString(e));
+      return -2;
+    }
+    configured = true;
+  }
+  const long long blocks = (long long)tiles_m * tiles_n;
+  LQ_REQUIRE(blocks < (1ll << 31), "linear: too many tiles");
+  LQ_REQUIRE(splits >= 1 && K % (BK * splits) == 0, "linear: the pipelined kernel needs K to be a multiple of %d",
+             BK * splits);
+  LQ_REQUIRE(splits == 1 || EPI == EPI_NONE, "linear: no epilogue on partial products");
+  kernel<<<dim3((int)blocks, splits), S::NW * 64, S::LDS_BYTES, stream>>>(
+      (const bf16_t*)A, lda, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, tiles_m, tiles_n, K / splits, split_stride);
+  LQ_CHECK_LAUNCH("linear(mfma pipelined)");
   return 0;
 }
 
@@ -442,16 +623,33 @@ int pick_skinny(const void* x, const void* w, void* out, int M, int N, int K, in
   return launch_skinny<16, MT, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
 }
 
+// The large pipelined tile pays once its tiles (times the shares of K) fill three quarters of the chip.
+inline bool fills_chip(long long blocks) { return blocks * 4 >= 3ll * lq_compute_units(); }
+
+// Shares of K for more than 64 rows: few tiles of 256 x 256 (a narrow weight matrix, a short prompt)
+// leave compute units idle; sharing K out over blocks fills them.
+int tiled_splits(int M, int N, int K) {
+  if (K % 64 != 0) return 1;
+  const long long t256 = (long long)lq_ceil_div(M, 256) * lq_ceil_div(N, 256);
+  int splits = 1;
+  while (splits < 8 && !fills_chip(t256 * splits) && K % (128 * splits) == 0 && K / (splits * 2) >= 1024) splits *= 2;
+  return splits;
+}
+
+int mfma_splits(int M, int N, int K) { return M <= 64 ? v3_splits(M, N, K) : tiled_splits(M, N, K); }
+
 template <int EPI, typename TO>
 int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
              int splits, long long split_stride, hipStream_t stream) {
   if (splits > 1) {
-    if (EPI != EPI_NONE || splits != v3_splits(M, N, K)) {
-      lq_set_error("linear: %d shares of K are not what this product takes (%d)", splits, v3_splits(M, N, K));
+    if (EPI != EPI_NONE || splits != mfma_splits(M, N, K)) {
+      lq_set_error("linear: %d shares of K are not what this product takes (%d)", splits, mfma_splits(M, N, K));
       return -1;
     }
     if (M <= 32) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
-    return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+    if (M <= 64) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride,
+                                                        stream);
   }
   // wide enough to give every compute unit a run of columns: the balanced kernel; else the simple one
   const bool wide = N >= 8 * lq_compute_units() && K >= 512;
@@ -467,10 +665,15 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
     if (wide) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     return pick_skinny<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
-  // the wider tile reuses each x fragment for twice the columns; it pays once there are enough tiles
-  // of it to fill every compute unit twice over
-  const long long wide_tiles = (long long)lq_ceil_div(M, 128) * lq_ceil_div(N, 256);
-  if (wide_tiles >= 2 * lq_compute_units()) return launch_tiled<2, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+  // the largest tile that still fills the chip: 256 x 256 (8 waves), 128 x 256 (4 waves, pipelined),
+  // then the register-staged kernels, which also take a K that is no multiple of 32
+  const long long t256 = (long long)lq_ceil_div(M, 256) * lq_ceil_div(N, 256);
+  const long long t128 = (long long)lq_ceil_div(M, 128) * lq_ceil_div(N, 256);
+  if (K % 64 == 0 && fills_chip(t256))
+    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+  if (K % 32 == 0 && t128 >= lq_compute_units())
+    return launch_pipelined<2, 2, 2, 4, 32, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+  if (t128 >= 2 * lq_compute_units()) return launch_tiled<2, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   return launch_tiled<2, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
 }
 
@@ -484,13 +687,23 @@ extern "C" int lq_debug_gemm_tiled(const void* x, const void* w, void* out, int 
   if (wm == 2 && wn == 4) return launch_tiled<2, 4, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
   if (wm == 4 && wn == 4) return launch_tiled<4, 4, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
   if (wm == 1 && wn == 2) return launch_tiled<1, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
+  // negative: the pipelined kernel; wm = -(stages), wn = -(variant)
+  if (wn == -1) return launch_pipelined<2, 2, 2, 4, 32, 3, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -2) return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -3) return launch_pipelined<4, 2, 2, 4, 32, 4, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -4) return launch_pipelined<4, 2, 2, 4, 32, 3, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -5) return launch_pipelined<2, 4, 4, 2, 32, 4, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -6)  // two shares of K: out holds two partial products
+    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 2, (long long)M * N, stream);
+  if (wn == -7)
+    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 4, (long long)M * N, stream);
   lq_set_error("no such tile");
   return -1;
 }
 
-// Whether the MFMA kernels take this problem (the caller falls back to the generic kernel if not).
-int lq_gemm_mfma_splits(int M, int N, int K) { return v3_splits(M, N, K); }
+int lq_gemm_mfma_splits(int M, int N, int K) { return mfma_splits(M, N, K); }
 
+// Whether the MFMA kernels take this problem (the caller falls back to the generic kernel if not).
 bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int lda, int ldw) {
   return in_dtype == LQ_BF16 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 &&
          ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;

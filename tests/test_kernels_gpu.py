@@ -112,6 +112,8 @@ def test_linear_float32(kn, m, n, k):
     (17, 256, 128), (32, 4096, 4096), (33, 515, 1000), (64, 130, 264), (64, 4096, 14336),  # skinny, more row tiles
     (65, 256, 128), (100, 300, 1000), (128, 128, 64), (257, 515, 4096),                   # tiled
     (2048, 1024, 512),
+    (1000, 12700, 192), (300, 49000, 64), (2048, 6144, 4096),     # pipelined, 256 x 256 tiles
+    (1000, 8200, 96), (130, 66000, 32), (2048, 4096, 4000),        # pipelined, 128 x 256 tiles
 ])
 def test_linear_bfloat16_matrix_cores(kn, out_dtype, m, n, k):
     x, w = rnd((m, k), 12, torch.bfloat16), rnd((n, k), 13, torch.bfloat16)
@@ -122,13 +124,14 @@ def test_linear_bfloat16_matrix_cores(kn, out_dtype, m, n, k):
     assert rel_err(out, want) < (1e-5 if out_dtype == torch.float32 else 5e-3)
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 4096, 4096), (17, 4096, 14336), (40, 2560, 2056), (33, 6144, 4096)])
+@pytest.mark.parametrize("m,n,k", [(64, 4096, 4096), (17, 4096, 14336), (40, 2560, 2056), (33, 6144, 4096),
+                                   (300, 4096, 4096), (2048, 4096, 14336), (65, 1000, 2048)])
 def test_linear_in_pieces_and_their_consumers(kn, m, n, k):
     """Few columns and several row tiles: K is shared out over blocks and the product comes as
     pieces; the norm, the add and the row gather that take such a delta add the pieces up."""
     pieces = kn.linear_pieces(torch.bfloat16, m, n, k)
     assert pieces > 1
-    assert kn.linear_pieces(torch.bfloat16, 8, n, k) == 1 and kn.linear_pieces(torch.float32, m, n, k) == 1
+    assert kn.linear_pieces(torch.bfloat16, 8, 4096, k) == 1 and kn.linear_pieces(torch.float32, m, n, k) == 1
     x, w = rnd((m, k), 40, torch.bfloat16), rnd((n, k), 41, torch.bfloat16)
     out = torch.full((pieces, m, n), float("nan"), dtype=torch.float32, device=DEV)
     kn.linear(x, w, out)
@@ -142,8 +145,9 @@ def test_linear_in_pieces_and_their_consumers(kn, m, n, k):
     with pytest.raises(KernelLibraryError):
         kn.linear(x, w, torch.empty((pieces + 1, m, n), dtype=torch.float32, device=DEV))
 
+    # the consumers' own work: the stream plus the exact sum of the pieces as they are
     res = rnd((m, n), 42)
-    summed = res.double().cpu() + want
+    summed = res.double().cpu() + out.double().sum(0).cpu()
     r1, normed = res.clone(), torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
     nw = rnd((n,), 43)
     kn.rmsnorm(r1, nw, 1e-5, normed, delta=out)
@@ -344,11 +348,12 @@ def test_rope_store_rotates_and_writes_the_right_rows(kn, dtype):
         < (1e-4 if dtype == torch.float32 else 0.2)
 
 
-@pytest.mark.parametrize("m", [1, 8, 16, 33, 64, 65, 300])
-@pytest.mark.parametrize("inner,k", [(16, 8), (328, 96), (1000, 264), (14336, 4096)])
+@pytest.mark.parametrize("m", [1, 8, 16, 33, 64, 65, 300, 400])
+@pytest.mark.parametrize("inner,k", [(16, 8), (328, 96), (1000, 264), (8200, 96), (14336, 4096)])
 def test_linear_with_fused_swiglu(kn, m, inner, k):
-    """One kernel for silu(x Wg^T) * (x Wu^T), with gate and up rows interleaved in groups of 8."""
-    if inner == 14336 and m > 64:
+    """One kernel for silu(x Wg^T) * (x Wu^T), with gate and up rows interleaved in groups of 8
+    (every kernel of the product has this epilogue: the GEMVs, the tiled and the pipelined ones)."""
+    if inner == 14336 and m == 65:
         m = 130
     x = rnd((m, k), 41, torch.bfloat16)
     gate, up = rnd((inner, k), 42, torch.bfloat16, 0.05), rnd((inner, k), 43, torch.bfloat16, 0.05)
