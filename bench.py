@@ -120,8 +120,11 @@ def main() -> int:
         engine.step([StepEntry(slot, random_prompt(2048), [2047])])
         engine.release(slot)
         slot = engine.new_sequence()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
         engine.step([StepEntry(slot, random_prompt(2048), [2047])])
         torch.cuda.synchronize()
+        print(f"[bench] prefill of 2048 tokens: {(time.perf_counter() - t) * 1e3:.2f} ms", file=sys.stderr, flush=True)
         return 0
     value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
     step_bytes = weight_bytes_per_step(config) + args.batch * ctx_mean * kv_bytes_per_token(config)

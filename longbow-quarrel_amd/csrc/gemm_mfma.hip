@@ -83,6 +83,48 @@ __device__ inline void tile_epilogue(f32x16 (&acc)[WM][WN], TO* __restrict__ C, 
     }
 }
 
+// The same for 16-bit outputs of a whole block, through LDS: the accumulator layout gives a lane one
+// value of a row at a time (2-byte stores, 64 bytes a row), so the block first lays its output tile
+// out in LDS, [BM][OUT_W] 16-bit, and then writes whole rows, 16 bytes a lane.  `tile` must hold
+// BM * OUT_W * 2 bytes and be free (every wave past its last LDS read: the caller's barrier).
+template <int WM, int WN, int BM, int BN, int EPI, int THREADS>
+__device__ inline void block_epilogue_16(f32x16 (&acc)[WM][WN], bf16_t* __restrict__ C, int ldc, int M, int N, int m0,
+                                         int n0, int wrow, int wcol, int lane, int tid, bf16_t* tile) {
+  constexpr int OUT_W = EPI == EPI_SWIGLU ? BN / 2 : BN;
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int col = wcol + j * 32 + (lane & 31);  // within the block tile
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = wrow + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (EPI == EPI_SWIGLU) {
+          const float up = __shfl(acc[i][j][e], lane + 8, 64);
+          if ((col & 15) < 8) tile[row * OUT_W + ((col >> 4) << 3) + (col & 7)] = f32_to_bf16(silu_mul(acc[i][j][e], up));
+        } else {
+          tile[row * OUT_W + col] = f32_to_bf16(acc[i][j][e]);
+        }
+      }
+    }
+  __syncthreads();
+  const int n_out = EPI == EPI_SWIGLU ? N / 2 : N, c0 = EPI == EPI_SWIGLU ? n0 / 2 : n0;
+  const bool vec = ldc % 8 == 0 && ((uintptr_t)C % 16) == 0;
+  constexpr int CPR = OUT_W / 8;  // 16-byte chunks a row
+  for (int c = tid; c < BM * CPR; c += THREADS) {
+    const int row = c / CPR, cc = (c % CPR) * 8;
+    const int grow = m0 + row, gcol = c0 + cc;
+    if (grow >= M || gcol >= n_out) continue;
+    bf16_t* dst = C + (long long)grow * ldc + gcol;
+    const bf16_t* src = tile + row * OUT_W + cc;
+    if (vec && gcol + 8 <= n_out) {
+      *(u32x4*)dst = *(const u32x4*)src;
+    } else {
+      for (int q = 0; q < 8 && gcol + q < n_out; ++q) dst[q] = src[q];
+    }
+  }
+}
+
 // ------------------------------------------------------------------ tiled
 constexpr int TBK = 64;           // k per stage
 constexpr int TLD = TBK + 8;      // padded LDS row, in elements (144 bytes: conflict-free b128 reads)
@@ -344,7 +386,15 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     for (int q = 0; q < STAGES; ++q)
       if (t + q < slabs) step(q, t + q);
   }
-  tile_epilogue<WM, WN, EPI, TO>(acc, C, ldc, M, N, m0 + wm * WM * 32, n0 + wn * WN * 32, lane);
+  if constexpr (sizeof(TO) == 2) {
+    constexpr int OUT_BYTES = S::BM * (EPI == EPI_SWIGLU ? S::BN / 2 : S::BN) * 2;
+    static_assert(OUT_BYTES <= S::LDS_BYTES, "the output tile must fit the stages");
+    __syncthreads();  // every wave is past its last fragment read
+    block_epilogue_16<WM, WN, S::BM, S::BN, EPI, S::NW * 64>(acc, C, ldc, M, N, m0, n0, wm * WM * 32, wn * WN * 32, lane,
+                                                             tid, (bf16_t*)plds);
+  } else {
+    tile_epilogue<WM, WN, EPI, TO>(acc, C, ldc, M, N, m0 + wm * WM * 32, n0 + wn * WN * 32, lane);
+  }
 }
 
 template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO>
