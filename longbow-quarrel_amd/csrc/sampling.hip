@@ -10,7 +10,9 @@
 //   sum passes r (:168-184).
 // Two things differ on purpose.  No sort: the kept set is a prefix of the descending order, so
 // it is found as a threshold on the 64-bit key (logit bits, then lower index first) by bisection
-// with block-wide counts and masses.  And the running sum of the draw walks the kept candidates
+// over counts and masses.  A histogram of the row first cuts off a short list of the largest keys
+// that surely holds the kept set (more than top_k keys, or mass past top_p); the bisection and the
+// draw then run on that list in LDS, and on the whole row only when no such list fits.  And the running sum of the draw walks the kept candidates
 // in index order, not in order of probability: the law of the drawn token is the same, which
 // token a given random number picks is not.
 // Sums are double with a fixed tree, so a sequence's draw does not depend on the batch.
@@ -19,6 +21,8 @@
 // the random numbers (counter-based: draw n of a sequence depends on key and n only) and a ring
 // of the last 64 token ids.
 #include "common.h"
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -42,6 +46,12 @@ __device__ inline unsigned long long shfl_xor_u64(unsigned long long v, int off)
   lo = __shfl_xor(lo, off, 64);
   hi = __shfl_xor(hi, off, 64);
   return ((unsigned long long)hi << 32) | lo;
+}
+
+__device__ inline double shfl_f64(double v, int src) {
+  const unsigned long long bits = (unsigned long long)__double_as_longlong(v);
+  const unsigned hi = __shfl((unsigned)(bits >> 32), src, 64), lo = __shfl((unsigned)bits, src, 64);
+  return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
 }
 
 __device__ inline double shfl_xor_f64(double v, int off) {
@@ -187,192 +197,483 @@ struct SampleArgs {
   double* kept_mass;  // optional, per row: mass of the kept set / total mass
 };
 
-// One pass over the row: how many keys are >= theta, their mass (if wanted) and the smallest of them.
+// One pass over a set of logits: how many keys are >= theta, their mass (if wanted) and the smallest of them.
 struct PassResult {
   long long count;
   double mass;
   unsigned long long kmin;
 };
 
-__device__ inline PassResult pass_over(const float* lr, int V, unsigned long long theta, float mx, float invT,
-                                       bool want_mass, unsigned long long* smu, double* smd) {
-  long long cnt = 0;
-  double mass = 0.0;
-  unsigned long long kmin = ~0ull;
-  for (int i = threadIdx.x; i < V; i += THREADS) {
-    const float v = lr[i];
-    const unsigned long long k = key_of(v, i);
-    if (k >= theta) {
-      ++cnt;
-      if (want_mass) mass += (double)expf((v - mx) * invT);
-      kmin = k < kmin ? k : kmin;
+// f(logit, index) for every logit of the row, 16 bytes a lane where the row's alignment allows; the
+// order in which a thread meets its elements depends on V and the row's address only.
+template <typename F>
+__device__ inline void for_each_logit(const float* lr, int V, F f) {
+  const int tid = threadIdx.x;
+  const int head = min(V, (int)(((16u - (unsigned)((uintptr_t)lr & 15u)) & 15u) / 4u));
+  if (tid < head) f(lr[tid], tid);
+  const int n4 = (V - head) / 4;
+  const f32x4* p4 = (const f32x4*)(lr + head);
+#pragma unroll 4
+  for (int j = tid; j < n4; j += THREADS) {
+    const f32x4 x = p4[j];
+    const int i = head + 4 * j;
+    f(x[0], i);
+    f(x[1], i + 1);
+    f(x[2], i + 2);
+    f(x[3], i + 3);
+  }
+  const int tail = head + 4 * n4 + tid;
+  if (tail < V) f(lr[tail], tail);
+}
+
+// The whole row in memory, all threads of the block.
+struct RowPass {
+  const float* lr;
+  int V;
+  float mx, invT;
+  unsigned long long* smu;
+  double* smd;
+  __device__ PassResult over(unsigned long long theta, bool want_mass) const {
+    long long cnt = 0;
+    double mass = 0.0;
+    unsigned long long kmin = ~0ull;
+    for_each_logit(lr, V, [&](float v, int i) {
+      const unsigned long long k = key_of(v, i);
+      if (k >= theta) {
+        ++cnt;
+        if (want_mass) mass += (double)expf((v - mx) * invT);
+        kmin = k < kmin ? k : kmin;
+      }
+    });
+    PassResult r;
+    r.count = block_sum_i64(cnt, smu);
+    r.mass = want_mass ? block_sum_f64(mass, smd) : 0.0;
+    r.kmin = block_min_u64(kmin, smu);
+    return r;
+  }
+  // largest logit bits below lo, if any
+  __device__ bool max_below(unsigned long long lo, unsigned long long& below) const {
+    unsigned long long loc = 0ull;  // bits + 1, so that 0 means none
+    for_each_logit(lr, V, [&](float v, int) {
+      const unsigned long long hk = (unsigned long long)ordered_bits(v);
+      if (hk < lo && hk + 1ull > loc) loc = hk + 1ull;
+    });
+    loc = block_max_u64(loc, smu);
+    below = loc - 1ull;
+    return loc > 0ull;
+  }
+};
+
+// A short list of (logit, index) in LDS, ascending by index, worked on by one wave: no barriers.
+struct ListPass {
+  const float* val;
+  const int* idx;
+  int n;
+  float mx, invT;
+  __device__ PassResult over(unsigned long long theta, bool want_mass) const {
+    const int lane = threadIdx.x & 63;
+    long long cnt = 0;
+    double mass = 0.0;
+    unsigned long long kmin = ~0ull;
+    for (int j = lane; j < n; j += 64) {
+      const float v = val[j];
+      const unsigned long long k = key_of(v, idx[j]);
+      if (k >= theta) {
+        ++cnt;
+        if (want_mass) mass += (double)expf((v - mx) * invT);
+        kmin = k < kmin ? k : kmin;
+      }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      cnt += (long long)shfl_xor_u64((unsigned long long)cnt, off);
+      mass += shfl_xor_f64(mass, off);
+      const unsigned long long o = shfl_xor_u64(kmin, off);
+      kmin = o < kmin ? o : kmin;
+    }
+    PassResult r;
+    r.count = cnt;
+    r.mass = mass;
+    r.kmin = kmin;
+    return r;
+  }
+  __device__ bool max_below(unsigned long long lo, unsigned long long& below) const {
+    const int lane = threadIdx.x & 63;
+    unsigned long long loc = 0ull;
+    for (int j = lane; j < n; j += 64) {
+      const unsigned long long hk = (unsigned long long)ordered_bits(val[j]);
+      if (hk < lo && hk + 1ull > loc) loc = hk + 1ull;
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const unsigned long long o = shfl_xor_u64(loc, off);
+      loc = o > loc ? o : loc;
+    }
+    below = loc - 1ull;
+    return loc > 0ull;
+  }
+};
+
+// The kept set is the longest allowed prefix of the descending order: at most k_limit members, all
+// above the floor, and without its last member not yet at the top_p mass.  As a set it is
+// {key >= theta}; allowed() is monotone in theta, so theta is found by bisection: first on the logit
+// bits (whole groups of equal logits) from lo_bits up, then, only if the group below the boundary has
+// several members, on the index bits inside that group.  `pass` must see every key >= lo_bits << 32,
+// and the set of all of them must not be allowed unless lo_bits is 0.
+template <typename P>
+__device__ inline unsigned long long find_theta(const P& pass, unsigned long long best, unsigned long long lo_bits,
+                                                long long k_limit, double e_floor, bool use_p, double p_mass) {
+  auto allowed = [&](unsigned long long theta) -> bool {
+    const PassResult r = pass.over(theta, use_p);
+    if (r.count == 0) return true;
+    const double e_min = (double)expf((from_ordered_bits((unsigned)(r.kmin >> 32)) - pass.mx) * pass.invT);
+    return r.count <= k_limit && e_min > e_floor && (!use_p || r.mass - e_min < p_mass);
+  };
+  unsigned long long lo = lo_bits, hi = best >> 32;
+  // the group of the maximum may itself be too large for k; then the index bisection below handles it
+  if (!allowed(hi << 32)) {
+    lo = hi = (best >> 32) + 1ull;  // nothing of the top group fits as a whole
+  } else {
+    while (lo < hi) {
+      const unsigned long long mid = lo + (hi - lo) / 2ull;
+      if (allowed(mid << 32))
+        hi = mid;
+      else
+        lo = mid + 1ull;
     }
   }
-  PassResult r;
-  r.count = block_sum_i64(cnt, smu);
-  r.mass = want_mass ? block_sum_f64(mass, smd) : 0.0;
-  r.kmin = block_min_u64(kmin, smu);
-  return r;
+  unsigned long long theta = lo << 32;  // 2^32 << 32 would need best >> 32 == 0xffffffff, a NaN: excluded
+  if (lo > lo_bits) {
+    unsigned long long below = 0ull;
+    if (pass.max_below(lo, below) && below >= lo_bits) {
+      const PassResult grp = pass.over(below << 32, false);
+      const PassResult above = pass.over(lo << 32, false);
+      if (grp.count - above.count > 1) {
+        // several equal logits: admit them one by one in index order while allowed;
+        // allowed(lo << 32) holds, allowed(below << 32) does not
+        unsigned long long a2 = (below << 32) + 1ull, b2 = lo << 32;
+        while (a2 < b2) {
+          const unsigned long long mid = a2 + (b2 - a2) / 2ull;
+          if (allowed(mid))
+            b2 = mid;
+          else
+            a2 = mid + 1ull;
+        }
+        theta = a2;
+      }
+    }
+  }
+  return theta;
 }
+
+// Histogram of the row over (max - logit): bin width chosen so that every candidate (p > 1e-10) falls
+// into the bins before the last.  Counts and masses are integers (mass in units of 2^-40), so that the
+// order of the atomic additions does not matter.
+constexpr int HIST_BINS = 1024;
+constexpr int LIST_CAP = 6144;   // entries of the short list in LDS
+constexpr double MASS_UNIT = 1099511627776.0;  // 2^40
 
 __global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a) {
   __shared__ unsigned long long smu[THREADS / 64];
   __shared__ double smd[THREADS / 64];
   __shared__ double scan[THREADS];
   __shared__ int winner;
-  const int row = blockIdx.x, tid = threadIdx.x;
+  __shared__ unsigned hist_count[HIST_BINS];
+  __shared__ unsigned long long hist_mass[HIST_BINS];
+  __shared__ float list_val[LIST_CAP];
+  __shared__ int list_idx[LIST_CAP];
+  __shared__ int wave_count[THREADS / 64 + 1];
+  __shared__ int cut_bin;
+  __shared__ unsigned long long theta_sh;
+  __shared__ int tok_sh, kept_sh;
+  __shared__ double total_sh;
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* lr = a.logits + (long long)row * a.ld;
   const int V = a.V;
   const float invT = a.inv_temperature;
 
   // maximum logit (as a key: also gives the arg-max)
   unsigned long long best = 0ull;
-  for (int i = tid; i < V; i += THREADS) {
-    const unsigned long long k = key_of(lr[i], i);
+  for_each_logit(lr, V, [&](float v, int i) {
+    const unsigned long long k = key_of(v, i);
     best = k > best ? k : best;
-  }
+  });
   best = block_max_u64(best, smu);
   const float mx = from_ordered_bits((unsigned)(best >> 32));
 
   // e_i = exp((l_i - max) / T) in 32-bit, sums in double; Z = sum e_i; candidates need p > 1e-10
   double zloc = 0.0;
-  for (int i = tid; i < V; i += THREADS) zloc += (double)expf((lr[i] - mx) * invT);
+  for_each_logit(lr, V, [&](float v, int) { zloc += (double)expf((v - mx) * invT); });
   const double Z = block_sum_f64(zloc, smd);
   const double e_floor = 1e-10 * Z;
-  long long ncand_loc = 0;
-  for (int i = tid; i < V; i += THREADS)
-    if ((double)expf((lr[i] - mx) * invT) > e_floor) ++ncand_loc;
-  const long long ncand = block_sum_i64(ncand_loc, smu);
-  const long long k_limit = (a.top_k > 0 && a.top_k < ncand) ? a.top_k : ncand;
   const bool use_p = a.top_p > 0.f && a.top_p < 1.f;
   const double p_mass = (double)a.top_p * Z;
 
-  // The kept set is the longest allowed prefix of the descending order: at most k_limit members,
-  // all above the floor, and without its last member not yet at the top_p mass.  As a set it is
-  // {key >= theta}; allowed() is monotone in theta, so theta is found by bisection: first on the
-  // logit bits (whole groups of equal logits), then, only if the group below the boundary has
-  // several members, on the index bits inside that group.
-  auto allowed = [&](unsigned long long theta) -> bool {
-    const PassResult r = pass_over(lr, V, theta, mx, invT, use_p, smu, smd);
-    if (r.count == 0) return true;
-    const double e_min = (double)expf((from_ordered_bits((unsigned)(r.kmin >> 32)) - mx) * invT);
-    return r.count <= k_limit && e_min > e_floor && (!use_p || r.mass - e_min < p_mass);
-  };
-  unsigned long long theta;
-  if (!use_p && k_limit == (long long)V) {
-    theta = 0ull;  // everything is kept
-  } else {
-    unsigned long long lo = 0ull, hi = best >> 32;  // allowed(hi << 32): the arg-max's group... checked below
-    // the group of the maximum may itself be too large for k; then the index bisection below handles it
-    if (!allowed(hi << 32)) {
-      lo = hi = (best >> 32) + 1ull;  // nothing of the top group fits as a whole
-    } else {
-      while (lo < hi) {
-        const unsigned long long mid = lo + (hi - lo) / 2ull;
-        if (allowed(mid << 32))
-          hi = mid;
-        else
-          lo = mid + 1ull;
-      }
-    }
-    theta = lo << 32;  // may be 2^32 << 32 = overflow only if best>>32 == 0xffffffff, i.e. +NaN: excluded
-    if (lo > 0ull) {
-      // the next group below the boundary: largest logit bits < lo
-      unsigned long long below = 0ull;
-      bool any = false;
-      {
-        unsigned long long loc = 0ull;
-        for (int i = tid; i < V; i += THREADS) {
-          const unsigned long long hk = (unsigned long long)ordered_bits(lr[i]);
-          if (hk < lo && hk + 1ull > loc) loc = hk + 1ull;  // store hk + 1 so that 0 means none
-        }
-        loc = block_max_u64(loc, smu);
-        any = loc > 0ull;
-        below = loc - 1ull;
-      }
-      if (any) {
-        const PassResult grp = pass_over(lr, V, below << 32, mx, invT, false, smu, smd);
-        const PassResult above = pass_over(lr, V, lo << 32, mx, invT, false, smu, smd);
-        if (grp.count - above.count > 1) {
-          // several equal logits: admit them one by one in index order while allowed
-          unsigned long long l2 = below << 32, h2 = lo << 32;  // allowed(h2) holds, allowed(l2) does not
-          // find the smallest allowed theta in (l2, h2]
-          unsigned long long a2 = l2 + 1ull, b2 = h2;
-          while (a2 < b2) {
-            const unsigned long long mid = a2 + (b2 - a2) / 2ull;
-            if (allowed(mid))
-              b2 = mid;
-            else
-              a2 = mid + 1ull;
-          }
-          theta = a2;
-        }
-      }
-    }
+  // candidates: their number, the smallest of them; and the histogram
+  for (int bin = tid; bin < HIST_BINS; bin += THREADS) {
+    hist_count[bin] = 0u;
+    hist_mass[bin] = 0ull;
   }
+  __syncthreads();
+  // a candidate has (max - l) / T < ln(1e10) + ln(Z) <= 23.03 + ln(V): all of them lie in bins < HIST_BINS - 1
+  const float span = (23.1f + logf((float)V)) / invT;
+  const float inv_width = (float)(HIST_BINS - 1) / span;
+  const bool select = a.top_k > 0 || use_p;
+  long long ncand_loc = 0;
+  unsigned long long cand_min = ~0ull;
+  for_each_logit(lr, V, [&](float v, int i) {
+    const float e = expf((v - mx) * invT);
+    if ((double)e > e_floor) {
+      ++ncand_loc;
+      const unsigned long long k = key_of(v, i);
+      cand_min = k < cand_min ? k : cand_min;
+    }
+    if (select) {
+      const float d = (mx - v) * inv_width;
+      const int bin = (d >= 0.f && d < (float)(HIST_BINS - 1)) ? (int)d : HIST_BINS - 1;  // NaN: the last bin
+      atomicAdd(&hist_count[bin], 1u);
+      atomicAdd(&hist_mass[bin], (unsigned long long)((double)e * MASS_UNIT));
+    }
+  });
+  const long long ncand = block_sum_i64(ncand_loc, smu);
+  cand_min = block_min_u64(cand_min, smu);
+  const long long k_limit = (a.top_k > 0 && a.top_k < ncand) ? a.top_k : ncand;
+  __syncthreads();
 
-  // the draw: running sum over the kept candidates in index order
-  const int chunk = (V + THREADS - 1) / THREADS;
-  const int i0 = tid * chunk, i1 = min(V, i0 + chunk);
-  double mine = 0.0;
-  long long cnt_loc = 0;
-  for (int i = i0; i < i1; ++i)
-    if (key_of(lr[i], i) >= theta) {
-      mine += (double)expf((lr[i] - mx) * invT);
-      ++cnt_loc;
+  // A cut in the histogram: the first bins that surely hold more than the kept set (more than top_k
+  // keys, or a mass past top_p by a margin and then one more non-empty bin).  The keys of these bins
+  // become a short list in LDS, on which the threshold is then found exactly.
+  if (tid == 0) {
+    int cut = -1;
+    if (select) {
+      unsigned long long cum_n = 0ull, cum_m = 0ull;
+      const unsigned long long m_need = (unsigned long long)(p_mass * (1.0 + 1e-9) * MASS_UNIT) + (unsigned long long)V + 1ull;
+      bool mass_passed = false;
+      for (int bin = 0; bin < HIST_BINS - 1; ++bin) {
+        const unsigned n_here = hist_count[bin];
+        if (mass_passed && n_here > 0u) {
+          cut = bin;
+          break;
+        }
+        cum_n += n_here;
+        cum_m += hist_mass[bin];
+        if (a.top_k > 0 && cum_n > (unsigned long long)a.top_k) {
+          cut = bin;
+          break;
+        }
+        if (use_p && cum_m >= m_need) mass_passed = true;
+      }
     }
-  scan[tid] = mine;
-  __syncthreads();
-  // inclusive prefix sums of scan[]: lane j of wave 0 sums its 16 entries serially, a wave scan
-  // gives each lane what lies before it
-  if (tid < 64) {
-    double run = 0.0;
-    for (int j = 0; j < THREADS / 64; ++j) {
-      run += scan[tid * (THREADS / 64) + j];
-      scan[tid * (THREADS / 64) + j] = run;
-    }
-    double incl = run;
-    for (int off = 1; off < 64; off <<= 1) {
-      const unsigned long long bits = (unsigned long long)__double_as_longlong(incl);
-      const unsigned hi32 = __shfl_up((unsigned)(bits >> 32), off, 64);
-      const unsigned lo32 = __shfl_up((unsigned)bits, off, 64);
-      const double o = __longlong_as_double((long long)(((unsigned long long)hi32 << 32) | lo32));
-      if (tid >= off) incl += o;
-    }
-    const double before = incl - run;
-    for (int j = 0; j < THREADS / 64; ++j) scan[tid * (THREADS / 64) + j] += before;
+    cut_bin = cut;
   }
-  if (tid == 0) winner = -1;
   __syncthreads();
-  const double total = scan[THREADS - 1];
-  const long long kept = block_sum_i64(cnt_loc, smu);
+  const int cut = cut_bin;
+  int n_list = 0;
+  if (cut >= 0) {
+    for (int bin = tid; bin <= cut; bin += THREADS) n_list += (int)hist_count[bin];
+    n_list = (int)block_sum_i64(n_list, smu);
+  }
+  const bool short_list = cut >= 0 && n_list <= LIST_CAP;
 
   const int slot = a.seq_slot[row];
   const unsigned long long ctr = (unsigned long long)a.rng_ctr[slot];
   const double u = uniform_of((unsigned long long)a.rng_key[slot], ctr);
-  const double r = u * total;
-  const double hi_incl = scan[tid];
-  const double lo_excl = hi_incl - mine;
-  if (cnt_loc > 0 && r >= lo_excl && r < hi_incl) {
-    double acc = lo_excl;
-    int tok = -1;
+
+  if (short_list) {
+    // the list, ascending by index: every wave owns a contiguous run of the row
+    const int head = min(V, (int)(((16u - (unsigned)((uintptr_t)lr & 15u)) & 15u) / 4u));
+    const int n4 = (V - head) / 4;
+    const int per_wave = (n4 + THREADS / 64 - 1) / (THREADS / 64);
+    const int j_begin = min(n4, wave * per_wave), j_end = min(n4, j_begin + per_wave);
+    const f32x4* p4 = (const f32x4*)(lr + head);
+    auto in_cut = [&](float v) -> bool {
+      const float d = (mx - v) * inv_width;
+      return d >= 0.f && d < (float)(HIST_BINS - 1) && (int)d <= cut;
+    };
+    for (int phase = 0; phase < 2; ++phase) {
+      int at = phase == 0 ? 0 : wave_count[wave];  // where this wave's next entry goes
+      auto put = [&](bool take, float v, int i, unsigned long long before_mask) {
+        const unsigned long long m = __ballot(take);
+        if (phase == 1 && take) {
+          const int pos = at + __popcll(m & before_mask);
+          list_val[pos] = v;
+          list_idx[pos] = i;
+        }
+        at += __popcll(m);
+      };
+      const unsigned long long lt = (1ull << lane) - 1ull;
+      if (wave == 0) {  // the unaligned head of the row
+        const bool has = lane < head;
+        const float v = has ? lr[lane] : 0.f;
+        put(has && in_cut(v), v, lane, lt);
+      }
+      for (int j0 = j_begin; j0 < j_end; j0 += 64) {
+        const int j = j0 + lane;
+        const bool has = j < j_end;
+        const f32x4 x = has ? p4[j] : (f32x4){0.f, 0.f, 0.f, 0.f};
+        const int i = head + 4 * j;
+        // index order: lane by lane, and a lane's four in turn
+        const bool t0 = has && in_cut(x[0]), t1 = has && in_cut(x[1]), t2 = has && in_cut(x[2]), t3 = has && in_cut(x[3]);
+        const int mine = (int)t0 + (int)t1 + (int)t2 + (int)t3;
+        int incl = mine;
+        for (int off = 1; off < 64; off <<= 1) {
+          const int o = __shfl_up(incl, off, 64);
+          if (lane >= off) incl += o;
+        }
+        if (phase == 1) {
+          int pos = at + incl - mine;
+          if (t0) { list_val[pos] = x[0]; list_idx[pos] = i; ++pos; }
+          if (t1) { list_val[pos] = x[1]; list_idx[pos] = i + 1; ++pos; }
+          if (t2) { list_val[pos] = x[2]; list_idx[pos] = i + 2; ++pos; }
+          if (t3) { list_val[pos] = x[3]; list_idx[pos] = i + 3; ++pos; }
+        }
+        at += __shfl(incl, 63, 64);
+      }
+      if (wave == THREADS / 64 - 1) {  // the row's last few
+        const int i = head + 4 * n4 + lane;
+        const bool has = i < V;
+        const float v = has ? lr[i] : 0.f;
+        put(has && in_cut(v), v, i, lt);
+      }
+      if (phase == 0) {
+        __syncthreads();
+        if (lane == 0) wave_count[wave + 1] = at;  // counts first, shifted by one
+        __syncthreads();
+        if (tid == 0) {
+          wave_count[0] = 0;
+          for (int w = 1; w <= THREADS / 64; ++w) wave_count[w] += wave_count[w - 1];
+        }
+        __syncthreads();
+      }
+    }
+    __syncthreads();
+    // one wave finds the threshold and draws; the list holds every key >= its smallest one
+    if (wave == 0) {
+      ListPass pass{list_val, list_idx, n_list, mx, invT};
+      unsigned long long lo_key = ~0ull;
+      for (int j = lane; j < n_list; j += 64) {
+        const unsigned long long k = key_of(list_val[j], list_idx[j]);
+        lo_key = k < lo_key ? k : lo_key;
+      }
+      for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long o = shfl_xor_u64(lo_key, off);
+        lo_key = o < lo_key ? o : lo_key;
+      }
+      const unsigned long long theta = find_theta(pass, best, lo_key >> 32, k_limit, e_floor, use_p, p_mass);
+      // the draw: running sum over the kept entries in index order, a contiguous run of the list a lane
+      const int chunk = (n_list + 63) / 64;
+      const int j0 = min(n_list, lane * chunk), j1 = min(n_list, j0 + chunk);
+      double mine = 0.0;
+      int cnt = 0;
+      for (int j = j0; j < j1; ++j)
+        if (key_of(list_val[j], list_idx[j]) >= theta) {
+          mine += (double)expf((list_val[j] - mx) * invT);
+          ++cnt;
+        }
+      double incl = mine;
+      for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long bits = (unsigned long long)__double_as_longlong(incl);
+        const unsigned hi32 = __shfl_up((unsigned)(bits >> 32), off, 64);
+        const unsigned lo32 = __shfl_up((unsigned)bits, off, 64);
+        const double o = __longlong_as_double((long long)(((unsigned long long)hi32 << 32) | lo32));
+        if (lane >= off) incl += o;
+      }
+      const double all = shfl_f64(incl, 63);  // the mass of the kept set
+      int kept = cnt;
+      for (int off = 32; off > 0; off >>= 1) kept += __shfl_xor(kept, off, 64);
+      const double r = u * all;
+      const double lo_excl = incl - mine;
+      int tok = -1;
+      if (cnt > 0 && r >= lo_excl && r < incl) {
+        double acc = lo_excl;
+        for (int j = j0; j < j1; ++j)
+          if (key_of(list_val[j], list_idx[j]) >= theta) {
+            acc += (double)expf((list_val[j] - mx) * invT);
+            tok = list_idx[j];
+            if (r < acc) break;
+          }
+      }
+      // at most one lane's range holds r
+      for (int off = 32; off > 0; off >>= 1) tok = max(tok, __shfl_xor(tok, off, 64));
+      if (lane == 0) {
+        tok_sh = tok;
+        kept_sh = kept;
+        total_sh = all;
+      }
+    }
+    __syncthreads();
+  } else {
+    // the row itself: when nothing is cut (all candidates are kept) or the list would not fit
+    unsigned long long theta;
+    if (!select) {
+      theta = ncand > 0 ? cand_min : 0ull;  // every candidate: the floor is the only rule
+    } else {
+      RowPass pass{lr, V, mx, invT, smu, smd};
+      theta = find_theta(pass, best, 0ull, k_limit, e_floor, use_p, p_mass);
+    }
+    // the draw: running sum over the kept candidates in index order
+    const int chunk = (V + THREADS - 1) / THREADS;
+    const int i0 = min(V, tid * chunk), i1 = min(V, i0 + chunk);
+    double mine = 0.0;
+    long long cnt_loc = 0;
     for (int i = i0; i < i1; ++i)
       if (key_of(lr[i], i) >= theta) {
-        acc += (double)expf((lr[i] - mx) * invT);
-        tok = i;
-        if (r < acc) break;
+        mine += (double)expf((lr[i] - mx) * invT);
+        ++cnt_loc;
       }
-    winner = tok;  // the ranges are disjoint: at most one thread's range holds r
+    scan[tid] = mine;
+    __syncthreads();
+    // inclusive prefix sums of scan[]: lane j of wave 0 sums its 16 entries serially, a wave scan
+    // gives each lane what lies before it
+    if (tid < 64) {
+      double run = 0.0;
+      for (int j = 0; j < THREADS / 64; ++j) {
+        run += scan[tid * (THREADS / 64) + j];
+        scan[tid * (THREADS / 64) + j] = run;
+      }
+      double incl = run;
+      for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long bits = (unsigned long long)__double_as_longlong(incl);
+        const unsigned hi32 = __shfl_up((unsigned)(bits >> 32), off, 64);
+        const unsigned lo32 = __shfl_up((unsigned)bits, off, 64);
+        const double o = __longlong_as_double((long long)(((unsigned long long)hi32 << 32) | lo32));
+        if (tid >= off) incl += o;
+      }
+      const double before = incl - run;
+      for (int j = 0; j < THREADS / 64; ++j) scan[tid * (THREADS / 64) + j] += before;
+    }
+    if (tid == 0) winner = -1;
+    __syncthreads();
+    const double total = scan[THREADS - 1];
+    const long long kept = block_sum_i64(cnt_loc, smu);
+    const double r = u * total;
+    const double hi_incl = scan[tid];
+    const double lo_excl = hi_incl - mine;
+    if (cnt_loc > 0 && r >= lo_excl && r < hi_incl) {
+      double acc = lo_excl;
+      int tok = -1;
+      for (int i = i0; i < i1; ++i)
+        if (key_of(lr[i], i) >= theta) {
+          acc += (double)expf((lr[i] - mx) * invT);
+          tok = i;
+          if (r < acc) break;
+        }
+      winner = tok;  // the ranges are disjoint: at most one thread's range holds r
+    }
+    __syncthreads();
+    if (tid == 0) {
+      tok_sh = winner;
+      kept_sh = (int)kept;
+      total_sh = total;
+    }
+    __syncthreads();
   }
-  __syncthreads();
   if (tid == 0) {
-    int tok = winner;
+    int tok = tok_sh;
     if (tok < 0) tok = (int)(0xffffffffu - (unsigned)(best & 0xffffffffull));  // r fell on a rounding seam
     a.out[row] = tok;
     a.rng_ctr[slot] = (long long)(ctr + 1ull);
     if (a.recent) push_recent(a.recent, a.recent_n, slot, tok);
-    if (a.kept_count) a.kept_count[row] = (int)kept;
-    if (a.kept_mass) a.kept_mass[row] = total / Z;
+    if (a.kept_count) a.kept_count[row] = kept_sh;
+    if (a.kept_mass) a.kept_mass[row] = total_sh / Z;
   }
 }
 
