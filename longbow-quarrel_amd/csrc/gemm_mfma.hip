@@ -268,12 +268,14 @@ struct PipeShape {
   static constexpr int ROW_BYTES = BK * 2;
   static constexpr int CPR = BK / 8;                        // 16-byte chunks a row
   static constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;     // a wave's transfer is 64 lanes x 16 bytes
-  static constexpr int A_DMA = BM / ROWS_PER_DMA / NW, W_DMA = BN / ROWS_PER_DMA / NW;
+  // a stage is BM rows of A, then BN rows of W: TRANSFERS runs of 1 KiB, dealt out over the waves (DMA
+  // each; where that does not come out even, the last run is fetched more than once)
+  static constexpr int TRANSFERS = (BM + BN) / ROWS_PER_DMA, DMA = (TRANSFERS + NW - 1) / NW;
   static constexpr int A_BYTES = BM * ROW_BYTES, STAGE_BYTES = (BM + BN) * ROW_BYTES;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static constexpr int KK = BK / 16;                        // 16-k steps a slab
-  static_assert(BM % (ROWS_PER_DMA * NW) == 0 && BN % (ROWS_PER_DMA * NW) == 0, "transfers must deal out evenly");
-  static_assert((A_DMA + W_DMA) * (STAGES - 1) < 64, "vmcnt has 6 bits");
+  static_assert(BM % ROWS_PER_DMA == 0 && BN % ROWS_PER_DMA == 0, "a transfer must not straddle A and W");
+  static_assert(DMA * (STAGES - 1) < 64, "vmcnt has 6 bits");
   // chunk position of chunk c in row r: rows that share a 256-byte bank row get different positions
   __device__ static int swizzle(int row) { return (row / (256 / ROW_BYTES)) & (CPR - 1); }
 };
@@ -297,30 +299,23 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / GN, wn = wave % GN;
 
-  // where this lane's 16 bytes of each transfer come from: transfer j of the wave fills the LDS
-  // chunks [(NW j + wave) * 64, + 64); chunk p is row p / CPR, position p % CPR
-  const bf16_t* pa[S::A_DMA];
-  const bf16_t* pw[S::W_DMA];
+  // where this lane's 16 bytes of each transfer come from: transfer x = NW j + wave fills the stage's
+  // chunks [64 x, 64 x + 64); chunk p is stage row p / CPR (A rows first), position p % CPR
+  const bf16_t* src[S::DMA];
+  int dst[S::DMA];
 #pragma unroll
-  for (int j = 0; j < S::A_DMA; ++j) {
-    const int p = (j * S::NW + wave) * 64 + lane, row = p / S::CPR, c = (p % S::CPR) ^ S::swizzle(row);
-    pa[j] = A + (long long)min(m0 + row, M - 1) * lda + k_begin + c * 8;
-  }
-#pragma unroll
-  for (int j = 0; j < S::W_DMA; ++j) {
-    const int p = (j * S::NW + wave) * 64 + lane, row = p / S::CPR, c = (p % S::CPR) ^ S::swizzle(row);
-    pw[j] = W + (long long)min(n0 + row, N - 1) * ldw + k_begin + c * 8;
+  for (int j = 0; j < S::DMA; ++j) {
+    const int x = min(j * S::NW + wave, S::TRANSFERS - 1);
+    const int p = x * 64 + lane, row = p / S::CPR, c = (p % S::CPR) ^ S::swizzle(row);
+    src[j] = (row < S::BM ? A + (long long)min(m0 + row, M - 1) * lda : W + (long long)min(n0 + row - S::BM, N - 1) * ldw) +
+             k_begin + c * 8;
+    dst[j] = x * 1024;
   }
   auto dma = [&](int stage, int k0) {
     unsigned char* base = plds + stage * S::STAGE_BYTES;
 #pragma unroll
-    for (int j = 0; j < S::A_DMA; ++j)
-      __builtin_amdgcn_global_load_lds(LQ_GLOBAL_PTR(pa[j] + k0), LQ_LDS_PTR(base + (j * S::NW + wave) * 1024), 16, 0,
-                                       0);
-#pragma unroll
-    for (int j = 0; j < S::W_DMA; ++j)
-      __builtin_amdgcn_global_load_lds(LQ_GLOBAL_PTR(pw[j] + k0),
-                                       LQ_LDS_PTR(base + S::A_BYTES + (j * S::NW + wave) * 1024), 16, 0, 0);
+    for (int j = 0; j < S::DMA; ++j)
+      __builtin_amdgcn_global_load_lds(LQ_GLOBAL_PTR(src[j] + k0), LQ_LDS_PTR(base + dst[j]), 16, 0, 0);
   };
 
   // fragment addresses within a 32-row group: row lane % 32, chunk 2 kk + lane / 32, swizzled
@@ -348,9 +343,9 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     // this wave's transfers of slab t have landed (those of the slabs behind it may still fly) ...
     const int behind = min(STAGES - 2, slabs - 1 - t);
     if (STAGES >= 4 && behind == 2)
-      LQ_WAIT_VMCNT(2 * (S::A_DMA + S::W_DMA));
+      LQ_WAIT_VMCNT(2 * S::DMA);
     else if (STAGES >= 3 && behind == 1)
-      LQ_WAIT_VMCNT(S::A_DMA + S::W_DMA);
+      LQ_WAIT_VMCNT(S::DMA);
     else
       LQ_WAIT_VMCNT(0);
     // ... and so have everyone's; and everyone is done reading slab t - 1, whose stage is filled next
@@ -715,12 +710,23 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
     if (wide) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     return pick_skinny<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
-  // the largest tile that still fills the chip: 256 x 256 (8 waves), 128 x 256 (4 waves, pipelined),
-  // then the register-staged kernels, which also take a K that is no multiple of 32
+  // the largest tile that still fills the chip: 256 rows by 256, 224 or 192 columns (8 waves), 128 x 256
+  // (4 waves, pipelined), then the register-staged kernels, which also take a K that is no multiple of 32
   const long long t256 = (long long)lq_ceil_div(M, 256) * lq_ceil_div(N, 256);
   const long long t128 = (long long)lq_ceil_div(M, 128) * lq_ceil_div(N, 256);
-  if (K % 64 == 0 && fills_chip(t256))
-    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+  if (K % 64 == 0 && fills_chip(t256)) {
+    // Tiles run in rounds of one a compute unit; a narrower tile can save a round or fill a round that
+    // a wider one leaves part empty.  Cost of a round relative to the 256-column tile, as measured.
+    const int cus = lq_compute_units(), tm = lq_ceil_div(M, 256);
+    const double c256 = 1.00 * lq_ceil_div(tm * lq_ceil_div(N, 256), cus);
+    const double c224 = 0.96 * lq_ceil_div(tm * lq_ceil_div(N, 224), cus);
+    const double c192 = 0.79 * lq_ceil_div(tm * lq_ceil_div(N, 192), cus);
+    if (c256 <= c224 && c256 <= c192)
+      return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    if (c224 <= c192)
+      return launch_pipelined<8, 1, 1, 7, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    return launch_pipelined<4, 2, 2, 3, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+  }
   if (K % 32 == 0 && t128 >= lq_compute_units())
     return launch_pipelined<2, 2, 2, 4, 32, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
   if (t128 >= 2 * lq_compute_units()) return launch_tiled<2, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
@@ -747,6 +753,9 @@ extern "C" int lq_debug_gemm_tiled(const void* x, const void* w, void* out, int 
     return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 2, (long long)M * N, stream);
   if (wn == -7)
     return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 4, (long long)M * N, stream);
+  if (wn == -8) return launch_pipelined<4, 2, 2, 3, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -9) return launch_pipelined<8, 1, 1, 7, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -10) return launch_pipelined<4, 2, 2, 3, 32, 4, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
   lq_set_error("no such tile");
   return -1;
 }
