@@ -7,6 +7,11 @@ bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int
 int lq_gemm_mfma(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K, int lda,
                  int ldw, int ldc, int epilogue, int splits, long long split_stride, hipStream_t stream);
 int lq_gemm_mfma_splits(int M, int N, int K);
+int lq_gemm_fused_parts(int M, int N, int K);
+int lq_gemm_residual(const void* act, const void* w, float* x, float* sq_out, const float* gain, void* scaled,
+                     int ld_scaled, int M, int N, int K, int lda, int ldw, int ldx, hipStream_t stream);
+int lq_gemm_scaled(const void* h, int ldh, const float* sq_parts, int n_parts, int width, float eps, const void* w,
+                   void* out, int out_dtype, int M, int N, int K, int ldw, int ldc, int swiglu, hipStream_t stream);
 
 // In how many shares of K lq_linear wants to compute this product (1: whole).  With s > 1 shares the
 // caller passes an output of s pieces, `split_stride` elements apart; their sum is the product, and
@@ -44,4 +49,42 @@ extern "C" int lq_linear_swiglu(const void* x, const void* w, void* out, int in_
   LQ_REQUIRE(lq_linear_swiglu_supported(in_dtype, N, K) && lq_gemm_mfma_accepts(x, w, in_dtype, K, lda, ldw),
              "linear+swiglu: needs bfloat16, 16-byte aligned rows, K %% 8 == 0 and N %% 16 == 0");
   return lq_gemm_mfma(x, w, out, out_dtype, M, N, K, lda, ldw, ldc, 1, 1, 0, stream);
+}
+
+// ------------------------------------------------------------------ the products around a norm (decoding)
+// A pre-norm block's x += act . w^T; out = rmsnorm(x) . w2^T in two kernels instead of three.  The first
+// adds into the float32 stream, leaves per-row sums of squares, a part per block, and the rows times the
+// norm's gain in bfloat16; the second multiplies those rows with w2 and scales each output row by
+// 1 / sqrt(mean(x^2) + eps) from the parts.  (The rows are rounded to bfloat16 before the division by the
+// root mean square, not after: the same relative rounding.)  lq_linear_fused_parts: the number of parts
+// the first leaves for [M, K] x [N, K]^T, or 0 when these kernels do not take the size (then the caller
+// uses the separate kernels).
+extern "C" int lq_linear_fused_parts(int dtype, int M, int N, int K) {
+  if (dtype != LQ_BF16) return 0;
+  return lq_gemm_fused_parts(M, N, K);
+}
+
+extern "C" int lq_linear_residual(const void* act, const void* w, float* x, float* sq_out, const float* gain,
+                                  void* scaled, int ld_scaled, int dtype, int M, int N, int K, int lda, int ldw,
+                                  int ldx, int parts, hipStream_t stream) {
+  LQ_REQUIRE(act && w && x && sq_out, "linear_residual: null pointer");
+  LQ_REQUIRE((gain == nullptr) == (scaled == nullptr) && (scaled == nullptr || ld_scaled >= N),
+             "linear_residual: a gain and a place for the scaled rows come together");
+  LQ_REQUIRE(lda >= K && ldw >= K && ldx >= N, "linear_residual: a row stride is smaller than its row");
+  LQ_REQUIRE(parts > 0 && parts == lq_linear_fused_parts(dtype, M, N, K),
+             "linear_residual: M=%d N=%d K=%d leaves %d parts, not %d", M, N, K, lq_linear_fused_parts(dtype, M, N, K),
+             parts);
+  LQ_REQUIRE(lq_gemm_mfma_accepts(act, w, dtype, K, lda, ldw), "linear_residual: operands are not aligned");
+  return lq_gemm_residual(act, w, x, sq_out, gain, scaled, ld_scaled, M, N, K, lda, ldw, ldx, stream);
+}
+
+extern "C" int lq_linear_scaled(const void* h, int ldh, const float* sq_parts, int parts, float eps, const void* w,
+                                void* out, int dtype, int out_dtype, int M, int N, int K, int ldw, int ldc,
+                                int swiglu, hipStream_t stream) {
+  LQ_REQUIRE(h && sq_parts && w && out, "linear_scaled: null pointer");
+  LQ_REQUIRE(parts > 0 && ldh >= K && ldw >= K && ldc >= (swiglu ? N / 2 : N), "linear_scaled: bad sizes");
+  LQ_REQUIRE(lq_linear_fused_parts(dtype, M, N, K) > 0 && (!swiglu || N % 16 == 0),
+             "linear_scaled: M=%d N=%d K=%d is not taken", M, N, K);
+  LQ_REQUIRE(lq_gemm_mfma_accepts(h, w, dtype, K, ldh, ldw), "linear_scaled: operands are not aligned");
+  return lq_gemm_scaled(h, ldh, sq_parts, parts, K, eps, w, out, out_dtype, M, N, K, ldw, ldc, swiglu, stream);
 }

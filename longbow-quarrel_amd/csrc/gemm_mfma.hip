@@ -55,7 +55,9 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
 // gate rows 8j..8j+7 and rows 16j+8..16j+15 the matching up rows, so that the lane holding gate
 // column c (c % 16 < 8) finds its up value 8 lanes further; it writes silu(gate) * up to
 // out[m][8j + c % 8], an [M, N / 2] matrix.
-enum { EPI_NONE = 0, EPI_SWIGLU = 1 };
+// EPI_RESIDUAL adds the product into C (the float32 residual stream, updated in place) and leaves, per
+// row, the sum of squares of the block's updated columns in a table, for the norm that follows.
+enum { EPI_NONE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 2 };
 
 __device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
@@ -517,16 +519,36 @@ constexpr int V3_MAXT = 8;  // tiles a block may own
 constexpr int v3_kb(int mt) { return mt <= 2 ? 8 / mt : 2; }
 constexpr int v3_kw(int mt) { return mt == 1 ? 16 : 8; }
 
-template <int KW, int MT, int EPI, typename TO>
+// A product whose rows are scaled afterwards by the RMS statistic of the norm that its input stands for:
+// the input holds x * gain (not yet divided by the root mean square), the rows' sums of squares come in
+// parts (sq_parts[row][part], what the product before left), and out = rstd(row) * (input . w^T).
+struct RowScale {
+  const float* sq_parts;  // [M][n_parts]
+  int n_parts;
+  int width;              // of the normalised rows
+  float eps;
+};
+
+// For EPI_RESIDUAL: where the sums of squares go, and optionally the next product's input.
+struct ResidualOut {
+  float* sq_out;          // [M][gridDim.x]
+  const float* gain;      // [N] or null
+  bf16_t* scaled;         // [M][ld_scaled]: bfloat16(x_new * gain), or null
+  int ld_scaled;
+};
+
+template <int KW, int MT, int EPI, typename TO, bool SCALED>
 __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16_t* __restrict__ X, int ldx,
                                                                       const bf16_t* __restrict__ W, int ldw,
                                                                       TO* __restrict__ C, int ldc, int M, int N,
                                                                       int K, int cols_per_block, int ks_per_wave,
-                                                                      long long split_stride) {
+                                                                      long long split_stride, RowScale scale,
+                                                                      ResidualOut res) {
   constexpr int KB = v3_kb(MT);
   constexpr int NBUF = MT == 1 ? 2 : 1;
   constexpr int VALS = MT * 4;  // accumulator values a lane holds per tile
   __shared__ float red[NBUF][KW][VALS * 64];
+  __shared__ float fresh_sh[EPI == EPI_RESIDUAL ? 16 : 1][EPI == EPI_RESIDUAL ? V3_MAXT * 16 : 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, c16 = lane & 15;
   const int col_begin = blockIdx.x * cols_per_block;
@@ -542,6 +564,20 @@ __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16
 #pragma unroll
   for (int m = 0; m < MT; ++m) xp[m] = X + (long long)min(m * 16 + c16, M - 1) * ldx;
   const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  // the parts of a row's sum of squares, asked for now and added up after the products
+  __shared__ float rstd_sh[16];
+  float sq_mine[4] = {0.f, 0.f, 0.f, 0.f};
+  if (SCALED) {
+    static_assert(!SCALED || MT == 1, "one row tile");
+    if (wave < M) {  // 16 waves: wave w holds row w
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int b = lane + 64 * j;
+        sq_mine[j] = b < scale.n_parts ? scale.sq_parts[(long long)wave * scale.n_parts + b] : 0.f;
+      }
+    }
+  }
 
   f32x4 acc[V3_MAXT][MT];
 #pragma unroll
@@ -577,6 +613,17 @@ __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16
       }
     }
   }
+  if (SCALED) {
+    static_assert(!SCALED || KW == 16, "a wave a row");
+    if (wave < M) {
+      // more than 256 parts: the rest now
+      float sum = (sq_mine[0] + sq_mine[1]) + (sq_mine[2] + sq_mine[3]);
+      for (int b = lane + 256; b < scale.n_parts; b += 64) sum += scale.sq_parts[(long long)wave * scale.n_parts + b];
+      for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+      if (lane == 0) rstd_sh[wave] = 1.0f / sqrtf(sum / (float)scale.width + scale.eps);
+    }
+    // the barrier of the first tile's reduction below also publishes rstd_sh
+  }
   // acc[t][m][e] = C[m * 16 + (lane / 16) * 4 + e][col_begin + 16 t + lane % 16], partial over this
   // wave's k.  The waves share out the (m, e) values of a tile and each sums its share over all waves,
   // in wave order.
@@ -596,14 +643,35 @@ __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16
 #pragma unroll
         for (int w = 0; w < KW; ++w) s += r[w][v * 64 + lane];
         const int row = (v >> 2) * 16 + g * 4 + (v & 3);
+        if (SCALED) s *= rstd_sh[min(row, M - 1)];
         if (EPI == EPI_SWIGLU) {
           const float up = __shfl(s, lane + 8, 64);
           if (c16 < 8 && row < M && col + 8 < col_end)
             store_out<TO>(C + (long long)row * ldc + ((col_begin + t * 16) >> 1) + c16, silu_mul(s, up));
+        } else if constexpr (EPI == EPI_RESIDUAL) {
+          static_assert(EPI != EPI_RESIDUAL || sizeof(TO) == 4, "the residual stream is float32");
+          float fresh = 0.f;
+          float* xr = (float*)C + (long long)row * ldc + col;
+          if (row < M && col < col_end) {
+            fresh = *xr + s;
+            *xr = fresh;
+            if (res.scaled) res.scaled[(long long)row * res.ld_scaled + col] = f32_to_bf16(fresh * res.gain[col]);
+          }
+          if (row < 16) fresh_sh[row][t * 16 + c16] = fresh;  // zero beyond the matrix
         } else {
           if (row < M && col < col_end) store_out<TO>(C + (long long)row * ldc + col, s);
         }
       }
+    }
+  }
+  if (EPI == EPI_RESIDUAL) {
+    // sum of squares of this block's columns of every row, in a fixed order: wave w takes row w
+    __syncthreads();
+    for (int r = wave; r < min(M, 16); r += KW) {
+      float sum = 0.f;
+      for (int c = lane; c < ntiles * 16; c += 64) sum += fresh_sh[r][c] * fresh_sh[r][c];
+      for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+      if (lane == 0) res.sq_out[(long long)r * gridDim.x + blockIdx.x] = sum;
     }
   }
 }
@@ -633,24 +701,29 @@ int v3_splits(int M, int N, int K) {
   return splits;
 }
 
-template <int MT, int EPI, typename TO>
-int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc,
-                     int splits, long long split_stride, hipStream_t stream) {
-  constexpr int KW = v3_kw(MT);
-  const int cus = lq_compute_units() / splits;
-  // equal runs of columns, in units of 16 (8 without the paired epilogue), at most V3_MAXT tiles each
-  const int unit = EPI == EPI_SWIGLU ? 16 : 8;
+// Runs of columns for the balanced kernel: equal, in units of 16 (8 without a paired epilogue), at most
+// V3_MAXT tiles each; -> columns a block, blocks
+inline void v3_runs(int N, int cus, int unit, int& cols, int& grid) {
   int blocks = cus;
-  int cols = lq_ceil_div(lq_ceil_div(N, blocks), unit) * unit;
+  cols = lq_ceil_div(lq_ceil_div(N, blocks), unit) * unit;
   while (cols > V3_MAXT * 16) {
     blocks += cus;
     cols = lq_ceil_div(lq_ceil_div(N, blocks), unit) * unit;
   }
-  const int grid = lq_ceil_div(N, cols);
+  grid = lq_ceil_div(N, cols);
+}
+
+template <int MT, int EPI, typename TO, bool SCALED = false>
+int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc,
+                     int splits, long long split_stride, hipStream_t stream, RowScale scale = RowScale(),
+                     ResidualOut res = ResidualOut()) {
+  constexpr int KW = v3_kw(MT);
+  int cols, grid;
+  v3_runs(N, lq_compute_units() / splits, EPI == EPI_SWIGLU ? 16 : 8, cols, grid);
   const int ksteps = lq_ceil_div(K, 32);
   const int ks_per_wave = lq_ceil_div(ksteps, KW * splits);
-  gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO><<<dim3(grid, splits), KW * 64, 0, stream>>>(
-      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, cols, ks_per_wave, split_stride);
+  gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO, SCALED><<<dim3(grid, splits), KW * 64, 0, stream>>>(
+      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, cols, ks_per_wave, split_stride, scale, res);
   LQ_CHECK_LAUNCH("linear(mfma skinny v3)");
   return 0;
 }
@@ -752,6 +825,50 @@ extern "C" int lq_debug_gemm_tiled(const void* x, const void* w, void* out, int 
 }
 
 int lq_gemm_mfma_splits(int M, int N, int K) { return mfma_splits(M, N, K); }
+
+// The decode pair around a norm.  `residual`: x[M, N] (float32) += act[M, K] . w[N, K]^T; sq_out[M][parts]
+// takes each row's sum of squares over a block's columns, and, with a gain, scaled[M, N] takes
+// bfloat16(x * gain), the input of the product after the norm.  `scaled`: out = rstd(row) * (h . w^T) with
+// rstd from those parts, optionally through the SwiGLU epilogue.  Both are the balanced kernel with one
+// row tile; lq_gemm_fused_parts says how many parts it leaves (0: this size is not taken).
+int lq_gemm_fused_parts(int M, int N, int K) {
+  if (M < 1 || M > 16 || !(N >= 8 * lq_compute_units() && K >= 512) || K % 8 != 0) return 0;
+  int cols, grid;
+  v3_runs(N, lq_compute_units(), 8, cols, grid);
+  return grid;
+}
+
+int lq_gemm_residual(const void* act, const void* w, float* x, float* sq_out, const float* gain, void* scaled,
+                     int ld_scaled, int M, int N, int K, int lda, int ldw, int ldx, hipStream_t stream) {
+  ResidualOut res;
+  res.sq_out = sq_out;
+  res.gain = gain;
+  res.scaled = (bf16_t*)scaled;
+  res.ld_scaled = ld_scaled;
+  return launch_skinny_v3<1, EPI_RESIDUAL, float>(act, w, x, M, N, K, lda, ldw, ldx, 1, 0, stream, RowScale(), res);
+}
+
+int lq_gemm_scaled(const void* h, int ldh, const float* sq_parts, int n_parts, int width, float eps, const void* w,
+                   void* out, int out_dtype, int M, int N, int K, int ldw, int ldc, int swiglu, hipStream_t stream) {
+  RowScale sc;
+  sc.sq_parts = sq_parts;
+  sc.n_parts = n_parts;
+  sc.width = width;
+  sc.eps = eps;
+  if (swiglu) {
+    if (out_dtype == LQ_BF16)
+      return launch_skinny_v3<1, EPI_SWIGLU, bf16_t, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, sc);
+    if (out_dtype == LQ_F32)
+      return launch_skinny_v3<1, EPI_SWIGLU, float, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, sc);
+  } else {
+    if (out_dtype == LQ_BF16)
+      return launch_skinny_v3<1, EPI_NONE, bf16_t, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, sc);
+    if (out_dtype == LQ_F32)
+      return launch_skinny_v3<1, EPI_NONE, float, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, sc);
+  }
+  lq_set_error("linear: unknown output dtype %d", out_dtype);
+  return -1;
+}
 
 // Whether the MFMA kernels take this problem (the caller falls back to the generic kernel if not).
 bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int lda, int ldw) {

@@ -100,7 +100,8 @@ class DecodeGraph:
         """Runs the body's allocations without launching, to learn the workspace size."""
         e = self.engine
 
-        queries = ("attention_workspace", "attention_folds_rope", "linear_swiglu_supported", "linear_pieces")
+        queries = ("attention_workspace", "attention_folds_rope", "linear_swiglu_supported", "linear_pieces",
+                   "linear_fused_parts")
 
         class _Null:
             """Answers the size and capability questions truthfully, launches nothing."""

@@ -199,6 +199,58 @@ class HipKernels:
                                        c_int(self._rows2d(w, "w")), c_int(ldc), c_int(pieces), c_longlong(stride),
                                        c_int(1 if self.force_generic else 0), self.stream))
 
+    # -- the two products around a norm, for a few rows (decoding): x += act . w^T leaves every row's
+    # sum of squares in parts, and the product after the norm normalises its input from them itself
+    def linear_fused_parts(self, dtype: torch.dtype, m: int, n: int, k: int) -> int:
+        """How many parts `linear_residual` leaves a row for [m, k] x [n, k]^T; 0: these kernels do
+        not take the size (use `linear` and `rmsnorm`)."""
+        if self.force_generic or dtype not in _DTYPE_CODE:
+            return 0
+        return int(self.lib.lq_linear_fused_parts(c_int(_DTYPE_CODE[dtype]), c_int(m), c_int(n), c_int(k)))
+
+    def linear_residual(self, act: torch.Tensor, w: torch.Tensor, x: torch.Tensor, sq_parts: torch.Tensor,
+                        gain: Optional[torch.Tensor] = None, scaled: Optional[torch.Tensor] = None) -> None:
+        """x[M, N] (float32, in place) += act[M, K] . w[N, K]^T; sq_parts[M, parts] (float32) takes, a part
+        per block of columns, the sums of squares of the updated rows; with gain [N] (float32),
+        scaled[M, N] takes (x * gain) in the dtype of act: the input of `linear_scaled`."""
+        self._dev(act, w, x, sq_parts, gain, scaled)
+        m, k = act.shape
+        n = w.shape[0]
+        if w.shape[1] != k or tuple(x.shape) != (m, n) or act.dtype != w.dtype:
+            raise KernelLibraryError(f"linear_residual: act {tuple(act.shape)}, w {tuple(w.shape)}, x {tuple(x.shape)} do not fit")
+        if x.dtype != torch.float32 or sq_parts.dtype != torch.float32 or sq_parts.dim() != 2 \
+                or sq_parts.shape[0] != m or not sq_parts.is_contiguous():
+            raise KernelLibraryError("linear_residual: x and sq_parts [M, parts] must be float32")
+        if (gain is None) != (scaled is None):
+            raise KernelLibraryError("linear_residual: gain and scaled come together")
+        if gain is not None and (gain.dtype != torch.float32 or gain.numel() != n or not gain.is_contiguous()
+                                 or tuple(scaled.shape) != (m, n) or scaled.dtype != act.dtype):
+            raise KernelLibraryError("linear_residual: gain must be float32 [N], scaled [M, N] in the dtype of act")
+        self._check(self.lib.lq_linear_residual(_ptr(act), _ptr(w), _ptr(x), _ptr(sq_parts), _ptr(gain), _ptr(scaled),
+                                                c_int(self._rows2d(scaled, "scaled") if scaled is not None else 0),
+                                                c_int(_code(act)), c_int(m), c_int(n), c_int(k),
+                                                c_int(self._rows2d(act, "act")), c_int(self._rows2d(w, "w")),
+                                                c_int(self._rows2d(x, "x")), c_int(sq_parts.shape[1]), self.stream))
+
+    def linear_scaled(self, h: torch.Tensor, sq_parts: torch.Tensor, eps: float, w: torch.Tensor,
+                      out: torch.Tensor, swiglu: bool = False) -> None:
+        """out[r] = (h[r] . w^T) / sqrt(mean + eps), mean being the sum of sq_parts[r, :] over K: with
+        h = x * gain this is rmsnorm(x) . w^T.  With `swiglu`, w holds interleaved gate and up rows and
+        out is [M, N / 2] (as `linear_swiglu`)."""
+        self._dev(h, sq_parts, w, out)
+        m, k = h.shape
+        n = w.shape[0]
+        n_out = n // 2 if swiglu else n
+        if w.shape[1] != k or tuple(out.shape) != (m, n_out) or h.dtype != w.dtype:
+            raise KernelLibraryError(f"linear_scaled: h {tuple(h.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+        if sq_parts.dtype != torch.float32 or sq_parts.dim() != 2 or sq_parts.shape[0] != m or not sq_parts.is_contiguous():
+            raise KernelLibraryError("linear_scaled: sq_parts [M, parts] must be float32")
+        self._check(self.lib.lq_linear_scaled(_ptr(h), c_int(self._rows2d(h, "h")), _ptr(sq_parts),
+                                              c_int(sq_parts.shape[1]), c_float(eps), _ptr(w), _ptr(out),
+                                              c_int(_code(w)), c_int(_code(out)), c_int(m), c_int(n), c_int(k),
+                                              c_int(self._rows2d(w, "w")), c_int(self._rows2d(out, "out")),
+                                              c_int(1 if swiglu else 0), self.stream))
+
     def linear_swiglu_supported(self, dtype: torch.dtype, rows_out: int, k: int) -> bool:
         """Whether `linear_swiglu` takes weights of this dtype with `rows_out` (= 2 I) rows and width k."""
         if self.force_generic or dtype not in _DTYPE_CODE:

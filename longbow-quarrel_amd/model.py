@@ -18,7 +18,7 @@ from typing import Dict, List, Mapping, Optional, Sequence
 
 import torch
 
-from .parts.base import (BLOCKS, MATRIX, NORMS, Block, BuildEnv, LayerCache, Norm, PartSpec,
+from .parts.base import (BLOCKS, MATRIX, NORMS, Block, BuildEnv, LayerCache, Norm, PartSpec, RowStats,
                          StepContext, TensorSpec, build_part, project)
 
 
@@ -108,11 +108,16 @@ class DecoderModel:
             if cache is not None and run.cache_of is not None:
                 cache = LayerCache(write=False, k=cache.k, v=cache.v, block_table=cache.block_table,
                                    block_size=cache.block_size, state=cache.state)
-            pending = self.blocks[run.layer].forward(x, pending, ctx, cache)
+            block = self.blocks[run.layer]
+            if block.takes_next_norm:
+                after = self.blocks[s.schedule[i + 1].layer].first_norm if i + 1 < len(s.schedule) else None
+                pending = block.forward(x, pending, ctx, cache, next_norm=after)
+            else:
+                pending = block.forward(x, pending, ctx, cache)
         if n_want == 0:
             return None
         picked = ctx.ws.alloc((n_want, s.width), torch.float32)
-        kn.gather_rows(x, want_rows, picked, delta=pending)
+        kn.gather_rows(x, want_rows, picked, delta=None if isinstance(pending, RowStats) else pending)
         normed = self.final_norm.forward(picked, ctx)
         logits = ctx.logits_out
         if logits is None:

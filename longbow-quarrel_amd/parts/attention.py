@@ -18,7 +18,7 @@ from typing import Dict, List, Mapping, Optional
 import torch
 
 from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mixer, PartSpec,
-                   StepContext, TensorSpec, build_part, project, project_delta)
+                   NormedRows, StepContext, TensorSpec, build_part, project, project_into, project_normed)
 
 
 @MIXERS.register("gqa_attention")
@@ -64,13 +64,19 @@ class GQAttention(Mixer):
     def cache_need(self) -> KVNeed:
         return KVNeed(self.kv_heads, self.head_dim, self.window)
 
-    def forward(self, h: torch.Tensor, ctx: StepContext, cache: Optional[LayerCache]) -> torch.Tensor:
+    takes_normed_rows = True
+    takes_residual_sink = True
+
+    def forward(self, h, ctx: StepContext, cache: Optional[LayerCache], sink=None) -> Optional[torch.Tensor]:
         if cache is None or cache.k is None:
             raise RuntimeError("attention needs a key/value cache")
         kn = ctx.kernels
         rows = h.shape[0]
         qkv = ctx.ws.alloc((rows, self.q_width + 2 * self.kv_width), ctx.dtype)
-        project(kn, ctx, h, self.w_qkv, qkv)
+        if not project_normed(kn, ctx, h, self.w_qkv, qkv):
+            if isinstance(h, NormedRows):
+                h = h.tensor(ctx)
+            project(kn, ctx, h, self.w_qkv, qkv)
         q = qkv[:, : self.q_width]
         k = qkv[:, self.q_width : self.q_width + self.kv_width]
         v = qkv[:, self.q_width + self.kv_width :]
@@ -99,4 +105,4 @@ class GQAttention(Mixer):
             kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
                          ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
                          self.scale, self.window, decode=ctx.decode, max_len=ctx.max_len, workspace=scratch)
-        return project_delta(kn, ctx, att, self.w_o)
+        return project_into(kn, ctx, att, self.w_o, sink)

@@ -244,12 +244,54 @@ class PositionEncoding(Part):
         raise NotImplementedError
 
 
+class RowStats:
+    """The residual stream is up to date and these are its rows' sums of squares, in parts
+    [rows, parts]: what a projection leaves that added its result into the stream itself.  If it
+    knew the norm that comes next, `scaled` holds x * that norm's gain in the run's dtype."""
+
+    def __init__(self, sq_parts: torch.Tensor, norm=None, scaled: Optional[torch.Tensor] = None) -> None:
+        self.sq_parts, self.norm, self.scaled = sq_parts, norm, scaled
+
+
+class NormedRows:
+    """Rows that are not normalised yet: the stream x, the norm that is due, x * gain (`scaled`) and
+    the rows' sums of squares.  A consumer whose first projection can divide its output rows by the
+    root mean square takes `scaled`, `sq_parts` and `eps`; anyone else calls tensor(ctx) and gets the
+    normalised rows."""
+
+    def __init__(self, x: torch.Tensor, norm, stats: RowStats) -> None:
+        self.x, self.norm = x, norm
+        self.scaled, self.sq_parts, self.eps = stats.scaled, stats.sq_parts, norm.eps
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    def tensor(self, ctx: "StepContext") -> torch.Tensor:
+        return self.norm.forward(self.x, ctx)
+
+
+class ResidualSink:
+    """Offered to a mixer or feed-forward that sets `takes_residual_sink`: it may add its result into
+    x itself (then it sets `stats` and returns None) instead of returning a delta.  `next_norm` is the
+    norm that the stream meets next, if the block knows it."""
+
+    def __init__(self, x: torch.Tensor, next_norm=None) -> None:
+        self.x, self.next_norm = x, next_norm
+        self.stats: Optional[RowStats] = None
+
+
 class Mixer(Part):
     """forward(h, ctx, cache) -> [rows, width], what the block adds to the residual stream.
 
     h are the normalised activations of the step's rows (packed; row r belongs
     to sequence ctx.row_seq[r] at position ctx.row_pos[r]).  A mixer must give
     the same result however a sequence's tokens are cut into steps."""
+
+    # Two optional shortcuts, both off unless a part sets the flag.  takes_normed_rows: h may be a
+    # NormedRows instead of a tensor.  takes_residual_sink: forward has a keyword `sink`.
+    takes_normed_rows = False
+    takes_residual_sink = False
 
     def cache_need(self):
         """KVNeed, StateNeed or None."""
@@ -262,6 +304,9 @@ class Mixer(Part):
 class FeedForward(Part):
     """forward(h, ctx) -> [rows, width]; row-independent."""
 
+    takes_normed_rows = False    # as for Mixer
+    takes_residual_sink = False
+
     def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
 
@@ -271,8 +316,14 @@ class Block(Part):
 
     forward(x, pending, ctx, cache) -> pending': x is the float32 residual
     stream [rows, width], updated in place; `pending` is a delta that still has
-    to be added to x (it lets the add ride on the next norm kernel).  The true
-    stream is x + pending."""
+    to be added to x (it lets the add ride on the next norm kernel): the true
+    stream is x + pending.  Or `pending` is a RowStats: x is up to date and its
+    rows' sums of squares are known.  A block that sets `takes_next_norm` is
+    also given `next_norm`, the first norm of the block that runs after it (or
+    None), and exposes its own as `first_norm`."""
+
+    takes_next_norm = False
+    first_norm = None
 
     mixer: Mixer
 
@@ -284,6 +335,34 @@ class Block(Part):
 def build_part(registry: Registry, spec: PartSpec, **extra):
     cls = registry.get(spec.kind)
     return cls(**dict(spec.params), **extra)
+
+
+def project_normed(kn, ctx: StepContext, h, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False) -> bool:
+    """out = rmsnorm(x) . w^T from a NormedRows without a norm kernel, if the kernels take the size."""
+    if not isinstance(h, NormedRows) or h.scaled is None or w.dtype != h.scaled.dtype:
+        return False
+    fused_parts = getattr(kn, "linear_fused_parts", None)
+    if fused_parts is None or fused_parts(w.dtype, h.scaled.shape[0], w.shape[0], w.shape[1]) <= 0:
+        return False
+    kn.linear_scaled(h.scaled, h.sq_parts, h.eps, w, out, swiglu=swiglu)
+    return True
+
+
+def project_into(kn, ctx: StepContext, act: torch.Tensor, w: torch.Tensor, sink: Optional[ResidualSink]):
+    """The last projection of a mixer or feed-forward: into the sink (-> None) where one is offered and
+    the kernels take the size, else as a delta (-> tensor)."""
+    if sink is not None and w.dtype == act.dtype:
+        fused_parts = getattr(kn, "linear_fused_parts", None)
+        rows = act.shape[0]
+        parts = fused_parts(act.dtype, rows, w.shape[0], w.shape[1]) if fused_parts else 0
+        if parts > 0:
+            sq = ctx.ws.alloc((rows, parts), torch.float32)
+            norm = sink.next_norm if getattr(sink.next_norm, "deferrable", False) else None
+            scaled = ctx.ws.alloc((rows, w.shape[0]), act.dtype) if norm is not None else None
+            kn.linear_residual(act, w, sink.x, sq, gain=norm.weight if norm is not None else None, scaled=scaled)
+            sink.stats = RowStats(sq, norm, scaled)
+            return None
+    return project_delta(kn, ctx, act, w)
 
 
 def project_delta(kn, ctx: StepContext, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:

@@ -1,15 +1,16 @@
 """The pre-norm decoder block: x += mixer(norm(x)); x += ffn(norm(x))
 (internal/device/metal.go:1326-1527: norm :1349, residual :1434, second norm
 :1451, residual :1474).  The residual stream stays float32; each add rides on
-the norm kernel that follows it."""
+the norm kernel that follows it, or, for the few rows of a decoding step, on the projection that
+produced it, which then also leaves the statistics for the norm that the next projection folds in."""
 from __future__ import annotations
 
 from typing import List, Mapping, Optional
 
 import torch
 
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, BuildEnv, LayerCache, PartSpec,
-                   StepContext, TensorSpec, build_part)
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, BuildEnv, LayerCache, NormedRows, PartSpec,
+                   ResidualSink, RowStats, StepContext, TensorSpec, build_part)
 
 
 @BLOCKS.register("prenorm")
@@ -35,9 +36,32 @@ class PreNormBlock(Block):
         for p in self.parts():
             p.bind(tensors, env)
 
-    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
-                cache: Optional[LayerCache]) -> Optional[torch.Tensor]:
-        h = self.mixer_norm.forward(x, ctx, delta=pending)
-        mixed = self.mixer.forward(h, ctx, cache)
-        h = self.ffn_norm.forward(x, ctx, delta=mixed)
+    takes_next_norm = True
+
+    @property
+    def first_norm(self):
+        return self.mixer_norm
+
+    @staticmethod
+    def _normed(norm, x: torch.Tensor, pending, ctx: StepContext, consumer):
+        """The rows for `consumer`: normalised now, or left for it to normalise where it can."""
+        if isinstance(pending, RowStats):
+            if consumer.takes_normed_rows and pending.norm is norm and pending.scaled is not None:
+                return NormedRows(x, norm, pending)
+            return norm.forward(x, ctx)
+        return norm.forward(x, ctx, delta=pending)
+
+    def forward(self, x: torch.Tensor, pending, ctx: StepContext, cache: Optional[LayerCache], next_norm=None):
+        h = self._normed(self.mixer_norm, x, pending, ctx, self.mixer)
+        if self.mixer.takes_residual_sink:
+            sink = ResidualSink(x, self.ffn_norm)
+            pending = self.mixer.forward(h, ctx, cache, sink=sink)
+            pending = sink.stats if pending is None else pending
+        else:
+            pending = self.mixer.forward(h, ctx, cache)
+        h = self._normed(self.ffn_norm, x, pending, ctx, self.ffn)
+        if self.ffn.takes_residual_sink:
+            sink = ResidualSink(x, next_norm)
+            pending = self.ffn.forward(h, ctx, sink=sink)
+            return sink.stats if pending is None else pending
         return self.ffn.forward(h, ctx)

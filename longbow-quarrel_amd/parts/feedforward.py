@@ -8,7 +8,8 @@ from typing import Dict, List, Mapping, Optional
 
 import torch
 
-from .base import FEED_FORWARDS, BuildEnv, FeedForward, StepContext, TensorSpec, project, project_delta
+from .base import (FEED_FORWARDS, BuildEnv, FeedForward, NormedRows, StepContext, TensorSpec, project, project_into,
+                   project_normed)
 
 
 @FEED_FORWARDS.register("swiglu")
@@ -46,14 +47,23 @@ class SwiGLU(FeedForward):
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = tensors[self.names["down"]].contiguous()
 
-    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+    takes_normed_rows = True
+    takes_residual_sink = True
+
+    def forward(self, h, ctx: StepContext, sink=None) -> Optional[torch.Tensor]:
         kn = ctx.kernels
         rows = h.shape[0]
         act = ctx.ws.alloc((rows, self.inner), ctx.dtype)
         if self.fused:
-            kn.linear_swiglu(h, self.w_gate_up, act)
+            if not project_normed(kn, ctx, h, self.w_gate_up, act, swiglu=True):
+                if isinstance(h, NormedRows):
+                    h = h.tensor(ctx)
+                kn.linear_swiglu(h, self.w_gate_up, act)
         else:
             gu = ctx.ws.alloc((rows, 2 * self.inner), torch.float32)
-            project(kn, ctx, h, self.w_gate_up, gu)
+            if not project_normed(kn, ctx, h, self.w_gate_up, gu):
+                if isinstance(h, NormedRows):
+                    h = h.tensor(ctx)
+                project(kn, ctx, h, self.w_gate_up, gu)
             kn.swiglu(gu, act)
-        return project_delta(kn, ctx, act, self.w_down)
+        return project_into(kn, ctx, act, self.w_down, sink)

@@ -14,6 +14,7 @@ from .base import NORMS, VECTOR32, BuildEnv, Norm, StepContext, TensorSpec
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     graph_safe = True
+    deferrable = True  # a consumer may apply it itself from x, weight, eps and the rows' sums of squares
 
     def __init__(self, width: int, eps: float, name: str) -> None:
         self.width = int(width)

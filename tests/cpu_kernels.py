@@ -34,6 +34,9 @@ class CpuKernels:
     def linear_pieces(self, dtype, m, n, k):
         return 1
 
+    def linear_fused_parts(self, dtype, m, n, k):
+        return 0
+
     def rmsnorm(self, x, weight, eps, out, delta=None):
         if delta is not None:
             x += self._whole(delta, x)

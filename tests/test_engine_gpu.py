@@ -192,6 +192,80 @@ def test_generation_in_bfloat16_graphs_and_direct_steps_agree(tmp_path_factory):
     assert alone.tokens[0] == batch.tokens[0]
 
 
+# wide enough for the kernels that fold a block's add and norm into the projections around them
+# (a few rows, at least 2 048 output columns): no size a power of two except the head size
+WIDE = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 2176, "intermediate_size": 2312,
+    "num_hidden_layers": 3, "num_attention_heads": 17, "num_key_value_heads": 1, "head_dim": 128,
+    "vocab_size": 1031, "max_position_embeddings": 256, "rms_norm_eps": 2e-6, "rope_theta": 40000.0,
+    "rope_scaling": None, "tie_word_embeddings": False, "torch_dtype": "bfloat16",
+    "bos_token_id": 1, "eos_token_id": 2,
+}
+
+
+def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory):
+    """A step of a few rows adds each projection's result into the stream in the projection itself
+    and leaves the norm to the projection that follows: against the plain implementation, as is the
+    same engine with these kernels switched off."""
+    folder = write_folder(tmp_path_factory.mktemp("wide"), WIDE, seed=3, std=0.03)
+    eng = lq.load_engine(folder, dtype="bfloat16", max_tokens=1024)
+    kn = eng.kernels
+    c, tensors = read_folder(folder)
+    ref = plain.PlainLlama(c, tensors)
+    reqs = [random_tokens(n, WIDE["vocab_size"], 300 + n) for n in (9, 21, 14)]
+    want = [ref.forward(r, plain.round_bf16) for r in reqs]
+    calls = {"residual": 0, "normed": 0}
+    res, nrm = kn.linear_residual, kn.linear_scaled
+
+    def counted(name, fn):
+        def f(*a, **k):
+            calls[name] += 1
+            return fn(*a, **k)
+        return f
+
+    def decode_all():
+        """prompts of 5 tokens in one step, then one token each until the shortest ends, and on"""
+        slots = [eng.new_sequence() for _ in reqs]
+        out = [[] for _ in reqs]
+        first = eng.step([StepEntry(s, r[:5], range(5)) for s, r in zip(slots, reqs)])
+        for i in range(len(reqs)):
+            out[i].append(first[5 * i : 5 * i + 5])
+        pos = 5
+        while any(pos < len(r) for r in reqs):
+            live = [i for i, r in enumerate(reqs) if pos < len(r)]
+            got = eng.step([StepEntry(slots[i], [reqs[i][pos]], [0]) for i in live])
+            for j, i in enumerate(live):
+                out[i].append(got[j : j + 1])
+            pos += 1
+        for s in slots:
+            eng.release(s)
+        return [torch.cat(o) for o in out]
+
+    kn.linear_residual, kn.linear_scaled = counted("residual", res), counted("normed", nrm)
+    try:
+        fused = decode_all()
+    finally:
+        kn.linear_residual, kn.linear_scaled = res, nrm
+    layers = WIDE["num_hidden_layers"]
+    steps = max(len(r) for r in reqs) - 5 + 1  # the prompts' step has 15 rows: few enough as well
+    assert calls["residual"] == 2 * layers * steps and calls["normed"] == (2 * layers - 1) * steps
+    for got, w in zip(fused, want):
+        assert rel_err(got, w) < TOL_BF16
+    parts = kn.linear_fused_parts
+    kn.linear_fused_parts = lambda *a: 0
+    try:
+        separate = decode_all()
+    finally:
+        kn.linear_fused_parts = parts
+    for got, w in zip(separate, want):
+        assert rel_err(got, w) < TOL_BF16
+    assert not any(torch.equal(a, b) for a, b in zip(fused, separate))  # they are two ways indeed
+    # and inside a captured step
+    g1 = lq.generate(eng, [r[:6] for r in reqs], 10, params=lq.SamplingParams(temperature=0.0), stop_ids=[], use_graphs=True)
+    g2 = lq.generate(eng, [r[:6] for r in reqs], 10, params=lq.SamplingParams(temperature=0.0), stop_ids=[], use_graphs=False)
+    assert g1.tokens == g2.tokens
+
+
 def test_command_line_generates_the_same_greedy_tokens(tmp_path_factory):
     eng, ref, act, reqs, want, folder = setup_case(tmp_path_factory, "a", "float32")
     prompt = reqs[1]

@@ -162,6 +162,51 @@ def test_linear_in_pieces_and_their_consumers(kn, m, n, k):
     assert rel_err(picked, summed[rows.long().cpu()]) < 1e-6
 
 
+@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("n,k,n2", [(4096, 4096, 6144), (4096, 14336, 28672), (2056, 520, 2304)])
+def test_products_around_a_norm(kn, m, n, k, n2):
+    """x += act . w^T with the rows' sums of squares left in parts and x * gain in bfloat16, then
+    rmsnorm(x) . w2^T as that times w2 with every output row divided by the root mean square:
+    against the add, the norm and the products one by one."""
+    parts = kn.linear_fused_parts(torch.bfloat16, m, n, k)
+    assert parts > 0 and kn.linear_fused_parts(torch.bfloat16, 17, n, k) == 0
+    act, w = rnd((m, k), 50, torch.bfloat16), rnd((n, k), 51, torch.bfloat16, 0.05)
+    gain, eps = rnd((n,), 53) + 1.0, 1e-5
+    x0 = rnd((m, n), 52)
+    x = x0.clone()
+    sq = torch.full((m, parts), float("nan"), dtype=torch.float32, device=DEV)
+    xg = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    kn.linear_residual(act, w, x, sq, gain=gain, scaled=xg)
+    want_x = x0.double().cpu() + act.double().cpu() @ w.double().cpu().t()
+    assert rel_err(x, want_x) < 1e-5
+    assert rel_err(sq.double().sum(1), (x.double() ** 2).sum(1)) < 1e-6  # of the float32 rows as they are
+    assert torch.equal(xg, (x * gain).to(torch.bfloat16))
+    x1, sq1 = x0.clone(), torch.empty_like(sq)
+    kn.linear_residual(act, w, x1, sq1)  # without a gain: the stream and the sums only
+    assert torch.equal(x1, x) and torch.equal(sq1, sq)
+
+    assert kn.linear_fused_parts(torch.bfloat16, m, n2, n) > 0
+    w2 = rnd((n2, n), 54, torch.bfloat16, 0.05)
+    xd = x.double().cpu()
+    rstd = 1.0 / torch.sqrt((xd * xd).mean(1, keepdim=True) + eps)
+    want = (xg.double().cpu() @ w2.double().cpu().t()) * rstd  # with the kernel's own rounding of x * gain
+    out32 = torch.empty((m, n2), dtype=torch.float32, device=DEV)
+    kn.linear_scaled(xg, sq, eps, w2, out32)
+    assert rel_err(out32, want) < 1e-5
+    out = torch.empty((m, n2), dtype=torch.bfloat16, device=DEV)
+    kn.linear_scaled(xg, sq, eps, w2, out)
+    assert rel_err(out, want) < 5e-3
+    # against the norm as the plain implementation rounds it (after the division, not before)
+    h = plain.round_bf16(plain.rms_norm(xd, gain.double().cpu(), eps))
+    assert rel_err(out32, h @ w2.double().cpu().t()) < 5e-3  # two bfloat16 roundings of the same rows
+    # the same through the SwiGLU epilogue (gate and up rows interleaved in groups of 8)
+    gate, up = w2[: n2 // 2], w2[n2 // 2 :]
+    wi = kn.interleave_gate_up(gate.contiguous(), up.contiguous())
+    act2 = torch.empty((m, n2 // 2), dtype=torch.bfloat16, device=DEV)
+    kn.linear_scaled(xg, sq, eps, wi, act2, swiglu=True)
+    assert rel_err(act2, plain.swiglu(want[:, : n2 // 2], want[:, n2 // 2 :])) < 5e-3
+
+
 def test_linear_bfloat16_odd_k_takes_the_generic_kernel(kn):
     x, w = rnd((9, 77), 14, torch.bfloat16), rnd((33, 77), 15, torch.bfloat16)
     out = torch.empty((9, 33), dtype=torch.float32, device=DEV)
