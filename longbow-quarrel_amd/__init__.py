@@ -5,6 +5,7 @@ One architecture (the Llama 3 dense decoder), one GPU, from a model folder
 kernels.
 """
 from . import models  # noqa: F401  (registers the architectures)
+from .api import QuarrelEngine, SamplerConfig, new_engine
 from .config import ConfigError, LlamaConfig, ModelConfig
 from .engine import Engine, GenerationResult, StepEntry, generate
 from .loading import load_engine, random_engine
@@ -14,5 +15,5 @@ from .weights import WeightError, write_model_folder
 
 __all__ = [
     "ConfigError", "LlamaConfig", "ModelConfig", "Engine", "StepEntry", "load_engine", "random_engine",
-    "GenerationResult", "generate", "SamplingParams", "register_architecture", "registered_architectures", "WeightError", "write_model_folder",
+    "GenerationResult", "generate", "SamplingParams", "QuarrelEngine", "SamplerConfig", "new_engine", "register_architecture", "registered_architectures", "WeightError", "write_model_folder",
 ]

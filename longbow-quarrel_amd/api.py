@@ -1,0 +1,76 @@
+"""The reference's programmatic interface, in Python's spelling: `NewEngine(path, cfg)`, `Infer`,
+`InferWithCallback`, `InferWithLogits`, `Close` (internal/engine/engine.go:380, 1273-1296) and
+`SamplerConfig{Temperature, TopK, TopP, RepPenalty, Seed}` (internal/engine/types_base.go:7-15).
+One sequence a call, as there; batches go through `generate`."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, List, Optional, Sequence, Tuple
+
+import torch
+
+from .engine.generate import EngineBackend, GenerationLoop
+from .loading import load_engine
+from .sampling import SamplingParams
+
+
+@dataclass(frozen=True)
+class SamplerConfig:
+    """Zero values mean what they mean in the reference: temperature 0 is greedy
+    (internal/engine/sampler.go:81-84), top_k <= 0 and top_p <= 0 or >= 1 are off (:309-339),
+    rep_penalty acts above 1 (:77-79).  Only the seed differs: 0 is a seed like any other here,
+    the reference takes the clock for it (:18-26)."""
+
+    temperature: float = 0.0
+    top_k: int = 0
+    top_p: float = 0.0
+    rep_penalty: float = 0.0
+    seed: int = 0
+
+    def params(self) -> SamplingParams:
+        return SamplingParams(temperature=self.temperature, top_k=max(0, self.top_k),
+                              top_p=self.top_p if 0.0 < self.top_p < 1.0 else 1.0,
+                              repetition_penalty=self.rep_penalty if self.rep_penalty > 1.0 else 1.0,
+                              seed=self.seed)
+
+
+class QuarrelEngine:
+    def __init__(self, path: str, dtype: str = "bfloat16", kv_cache_size: int = 2048,
+                 device: str = "cuda:0") -> None:
+        """`kv_cache_size`: tokens the cache holds (the reference's `KVCacheSize`, engine.go:388)."""
+        self.engine = load_engine(path, dtype=dtype, max_tokens=kv_cache_size, max_slots=1, device=device)
+
+    def _run(self, tokens: Sequence[int], n: int, cfg: Optional[SamplerConfig],
+             callback: Optional[Callable[[int], None]], keep_logits: bool) -> Tuple[List[int], Optional[torch.Tensor]]:
+        backend = EngineBackend(self.engine, (cfg or SamplerConfig()).params(), use_graphs=not keep_logits)
+        backend.keep_logits = keep_logits
+        try:
+            cb = (lambda _request, token: callback(token)) if callback is not None else None
+            out = GenerationLoop(backend, max_batch=1).run([list(tokens)], n, tuple(self.engine.model.spec.stop_ids),
+                                                           False, cb)
+            return out.tokens[0], backend.last_logits
+        finally:
+            backend.close()
+
+    def infer(self, tokens: Sequence[int], n: int, sampler_config: Optional[SamplerConfig] = None) -> List[int]:
+        """Up to n new ids after the prompt; the prompt is not returned (engine.go:1273-1276)."""
+        return self._run(tokens, n, sampler_config, None, False)[0]
+
+    def infer_with_callback(self, tokens: Sequence[int], n: int, sampler_config: Optional[SamplerConfig],
+                            callback: Callable[[int], None]) -> List[int]:
+        """`callback(id)` for every generated id as it is made (engine.go:1287-1296)."""
+        return self._run(tokens, n, sampler_config, callback, False)[0]
+
+    def infer_with_logits(self, tokens: Sequence[int], n: int,
+                          sampler_config: Optional[SamplerConfig] = None) -> Tuple[List[int], torch.Tensor]:
+        """The ids, and the float32 logits [vocab] that the last of them was drawn from, as the model
+        gave them (before the repetition penalty) (engine.go:1278-1285)."""
+        ids, logits = self._run(tokens, n, sampler_config, None, True)
+        return ids, logits[0]
+
+    def close(self) -> None:
+        self.engine = None
+
+
+def new_engine(path: str, **options) -> QuarrelEngine:
+    return QuarrelEngine(path, **options)

@@ -142,6 +142,8 @@ class EngineBackend:
         self.use_graphs = use_graphs and engine.device.type == "cuda" and engine.graph_safe
         self.graphs: Dict[tuple, DecodeGraph] = {}
         self.current: Optional[DecodeGraph] = None
+        self.keep_logits = False  # direct steps only: a copy of each step's logits before sampling changes them
+        self.last_logits: Optional[torch.Tensor] = None
 
     # ---- what the loop asks ------------------------------------------------------------
     def free_blocks(self) -> int:
@@ -175,6 +177,8 @@ class EngineBackend:
         e = self.engine
 
         def body():
+            if self.keep_logits:
+                self.last_logits = logits.clone()
             seq_slot = torch.tensor(list(slots), dtype=torch.int32).to(e.device)
             out = torch.empty(len(slots), dtype=torch.int32, device=e.device)
             self.sampler.sample(logits, seq_slot, out)

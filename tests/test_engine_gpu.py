@@ -266,6 +266,25 @@ def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory
     assert g1.tokens == g2.tokens
 
 
+def test_the_reference_style_interface(tmp_path_factory):
+    """new_engine / infer / infer_with_callback / infer_with_logits / close (internal/engine/engine.go:380,
+    1273-1296) give what `generate` gives for one sequence."""
+    eng, ref, act, reqs, want, folder = setup_case(tmp_path_factory, "b", "float32")
+    prompt = reqs[2][:12]
+    q = lq.new_engine(folder, dtype="float32", kv_cache_size=256)
+    greedy = lq.generate(eng, [prompt], 9, lq.SamplingParams(), stop_ids=[5, 7]).tokens[0]
+    assert q.infer(prompt, 9) == greedy == q.infer(prompt, 9, lq.SamplerConfig())
+    seen = []
+    assert q.infer_with_callback(prompt, 9, None, seen.append) == greedy and seen == greedy
+    ids, logits = q.infer_with_logits(prompt, 9)
+    assert ids == greedy and logits.shape == (TINY_B["vocab_size"],)
+    whole = ref.forward(prompt + greedy[:-1], plain.identity)
+    assert rel_err(logits, whole[-1]) < TOL_F32  # the logits the last id was taken from
+    cfg = lq.SamplerConfig(temperature=0.8, top_k=40, top_p=0.95, rep_penalty=1.1, seed=4)
+    assert q.infer(prompt, 9, cfg) == lq.generate(eng, [prompt], 9, cfg.params(), stop_ids=[5, 7]).tokens[0]
+    q.close()
+
+
 def test_command_line_generates_the_same_greedy_tokens(tmp_path_factory):
     eng, ref, act, reqs, want, folder = setup_case(tmp_path_factory, "a", "float32")
     prompt = reqs[1]
