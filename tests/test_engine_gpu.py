@@ -266,6 +266,50 @@ def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory
     assert g1.tokens == g2.tokens
 
 
+LONG = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermediate_size": 264,
+    "num_hidden_layers": 2, "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 128,
+    "vocab_size": 331, "max_position_embeddings": 4096, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 512},
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "bos_token_id": 1, "eos_token_id": 2,
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_sequence_longer_than_one_split_of_decode_attention(tmp_path_factory, dtype):
+    """1 300 tokens with the 8B head shape: the prompt in unequal cuts (many cache blocks a row tile),
+    then tokens one by one across the 1 024-key split boundary (two splits and their merge), with a
+    short sequence decoding in the same batch."""
+    folder = write_folder(tmp_path_factory.mktemp(f"long_{dtype}"), LONG, seed=9, std=0.08)
+    c, tensors = read_folder(folder)
+    ref = plain.PlainLlama(c, tensors)
+    act = plain.identity if dtype == "float32" else plain.round_bf16
+    n, head = 1300, 1010
+    req = random_tokens(n, LONG["vocab_size"], 77)
+    short = req[500:560]
+    want, want_short = ref.forward(req, act), ref.forward(short, act)
+    eng = lq.load_engine(folder, dtype=dtype, max_tokens=2048)
+    a, b = eng.new_sequence(), eng.new_sequence()
+    got = [eng.step([StepEntry(a, req[lo:hi], range(hi - lo))]) for lo, hi in ((0, 700), (700, 701), (701, head))]
+    eng.step([StepEntry(b, short[:20], [])])
+    got_short = []
+    for i in range(head, n):
+        entries = [StepEntry(a, [req[i]], [0])]
+        j = 20 + i - head
+        if j < len(short):
+            entries.append(StepEntry(b, [short[j]], [0]))
+        out = eng.step(entries)
+        got.append(out[:1])
+        if j < len(short):
+            got_short.append(out[1:2])
+    got, got_short = torch.cat(got), torch.cat(got_short)
+    assert rel_err(got[:head], want[:head]) < tol(dtype)
+    assert rel_err(got[head:], want[head:]) < tol(dtype)
+    assert rel_err(got[1020:1030], want[1020:1030]) < tol(dtype)  # the rows around the split boundary
+    assert rel_err(got_short, want_short[20:]) < tol(dtype)
+
+
 def test_the_reference_style_interface(tmp_path_factory):
     """new_engine / infer / infer_with_callback / infer_with_logits / close (internal/engine/engine.go:380,
     1273-1296) give what `generate` gives for one sequence."""
