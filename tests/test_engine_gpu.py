@@ -260,6 +260,12 @@ def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory
     for got, w in zip(separate, want):
         assert rel_err(got, w) < TOL_BF16
     assert not any(torch.equal(a, b) for a, b in zip(fused, separate))  # they are two ways indeed
+    # a prompt long enough for the tiled matrix-core kernels and their K-shared products
+    long_prompt = random_tokens(300, WIDE["vocab_size"], 9)
+    s = eng.new_sequence()
+    got = eng.step([StepEntry(s, long_prompt, range(300))])
+    eng.release(s)
+    assert rel_err(got, ref.forward(long_prompt, plain.round_bf16)) < TOL_BF16
     # and inside a captured step
     g1 = lq.generate(eng, [r[:6] for r in reqs], 10, params=lq.SamplingParams(temperature=0.0), stop_ids=[], use_graphs=True)
     g2 = lq.generate(eng, [r[:6] for r in reqs], 10, params=lq.SamplingParams(temperature=0.0), stop_ids=[], use_graphs=False)
