@@ -64,8 +64,14 @@ __device__ inline unsigned pack_bf16(float lo, float hi) {
 // probability that small is worth)
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// One chunk of 32 keys for one query tile: from the raw score tiles s[2] (S^T, lane holds keys
-// (lane/16)*4 + e of each 16-key tile for column lane%16) to the packed probabilities, updating the
+// Which key of a 32-key chunk row r of score tile j stands for: the rows are dealt out so that the
+// eight probabilities a lane ends up with (rows (lane/16)*4 + e of both tiles) belong to eight
+// consecutive keys, (lane/16)*8 .. +7: the second product then takes its V^T operand as one
+// 16-byte run of keys.
+__device__ inline int chunk_key(int j, int r) { return (r >> 2) * 8 + j * 4 + (r & 3); }
+
+// One chunk of 32 keys for one query tile: from the raw score tiles s[2] (S^T, lane holds rows
+// (lane/16)*4 + e of each 16-row tile, i.e. keys (lane/16)*8 + 4 j + e, for column lane%16) to the packed probabilities, updating the
 // running maximum m (log2 domain, scores scaled by c = scale * log2 e) and normaliser share l.
 // Returns the factor the output accumulator has to be multiplied with (1 if the maximum stayed).
 // `masked` is wave-uniform: false when every key of the chunk is visible to every column.
@@ -82,7 +88,7 @@ __device__ inline float softmax_chunk(const f32x4 (&s)[2], float c, bool masked,
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int t = t0 + 16 * j + g * 4 + e;
+        const int t = t0 + g * 8 + j * 4 + e;
         if (!(col_valid && t >= lo && t <= pos)) sv[j * 4 + e] = -INFINITY;
       }
   }
@@ -135,12 +141,12 @@ struct AttnArgs {
   const float* cs;
 };
 
-// One chunk's operands as they come from memory: 16 bytes a lane for each K fragment, two 8-byte
-// pieces a lane for each V^T fragment.
+// One chunk's operands as they come from memory: 16 bytes a lane for each K fragment and for each
+// V^T fragment.
 template <int HD>
 struct ChunkRegs {
   u32x4 k[2][HD / 32];
-  u32x2 v[HD / 16][2];
+  u32x4 v[HD / 16];
 };
 
 template <int HD>
@@ -151,13 +157,12 @@ __device__ inline void load_chunk(const AttnArgs& a, int kvh, long long blk, int
   for (int j = 0; j < 2; ++j)
 #pragma unroll
     for (int kk = 0; kk < HD / 32; ++kk)
-      r.k[j][kk] = *(const u32x4*)(kb + (16 * j + c16) * HD + kk * 32 + g * 8);
+      r.k[j][kk] = *(const u32x4*)(kb + chunk_key(j, c16) * HD + kk * 32 + g * 8);
   const bf16_t* vb = a.vcache + ((blk * a.nkv + kvh) * (long long)HD) * BS + koff;
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) {
     const bf16_t* vr = vb + (long long)(dt * 16 + c16) * BS;
-    r.v[dt][0] = *(const u32x2*)(vr + g * 4);
-    r.v[dt][1] = *(const u32x2*)(vr + 16 + g * 4);
+    r.v[dt] = *(const u32x4*)(vr + g * 8);
   }
 }
 
@@ -199,18 +204,14 @@ __device__ inline void attend(const AttnArgs& a, QTiles<HD, QT>& w, int kvh, con
     }
     // values of keys that were never written must not reach the product (0 * garbage may be NaN)
     if (t0 + 31 > t_written) {
-      const int ta = t0 + g * 4, tb = t0 + 16 + g * 4;
+      const int ta = t0 + g * 8;  // this lane's eight keys
 #pragma unroll
-      for (int dt = 0; dt < HD / 16; ++dt) {
-        if (ta + 0 > t_written) cur.v[dt][0][0] &= 0xffff0000u;
-        if (ta + 1 > t_written) cur.v[dt][0][0] &= 0x0000ffffu;
-        if (ta + 2 > t_written) cur.v[dt][0][1] &= 0xffff0000u;
-        if (ta + 3 > t_written) cur.v[dt][0][1] &= 0x0000ffffu;
-        if (tb + 0 > t_written) cur.v[dt][1][0] &= 0xffff0000u;
-        if (tb + 1 > t_written) cur.v[dt][1][0] &= 0x0000ffffu;
-        if (tb + 2 > t_written) cur.v[dt][1][1] &= 0xffff0000u;
-        if (tb + 3 > t_written) cur.v[dt][1][1] &= 0x0000ffffu;
-      }
+      for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (ta + 2 * e > t_written) cur.v[dt][e] &= 0xffff0000u;
+          if (ta + 2 * e + 1 > t_written) cur.v[dt][e] &= 0x0000ffffu;
+        }
     }
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
@@ -235,14 +236,8 @@ __device__ inline void attend(const AttnArgs& a, QTiles<HD, QT>& w, int kvh, con
           for (int e = 0; e < 4; ++e) w.o[qt][dt][e] *= alpha;
       }
 #pragma unroll
-      for (int dt = 0; dt < HD / 16; ++dt) {
-        u32x4 vv;
-        vv[0] = cur.v[dt][0][0];
-        vv[1] = cur.v[dt][0][1];
-        vv[2] = cur.v[dt][1][0];
-        vv[3] = cur.v[dt][1][1];
-        w.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vv), pb, w.o[qt][dt], 0, 0, 0);
-      }
+      for (int dt = 0; dt < HD / 16; ++dt)
+        w.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.v[dt]), pb, w.o[qt][dt], 0, 0, 0);
     }
   }
 }
@@ -264,7 +259,8 @@ __device__ inline void init_tiles(QTiles<HD, QT>& w) {
 // V^T [HD][64] from memory into padded LDS (next block's copy in registers while the current one is
 // multiplied), and every wave reads its MFMA operands from there, so a key is fetched once for
 // all the heads that share it.  LDS rows are padded (K: +16 bytes, V^T: +16 bytes) so that the
-// operand reads of a quarter wave fall into distinct banks.
+// operand reads of a quarter wave fall into distinct banks.  Keys lie in LDS in the order the score
+// tiles read them (chunk_key).
 template <int HD>
 struct RowsLds {
   static constexpr int K_STRIDE = HD * 2 + 16;   // bytes per key row
@@ -276,7 +272,7 @@ struct RowsLds {
 };
 
 template <int HD, int QT, int NW>
-__global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_rows_kernel(AttnArgs a, int heads_per_block_group) {
+__global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_rows_kernel(AttnArgs a, int heads_per_block_group) {
   using L = RowsLds<HD>;
   constexpr int ROWS = QT * 16;
   constexpr int THREADS = NW * 64;
@@ -355,8 +351,11 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_rows_kernel
     for (int i = 0; i < PER_THREAD; ++i) {
       const int pc = tid + i * THREADS;
       if (pc < L::PIECES) {
+        // keys go to the row their score tile reads them from: row 16 j + r holds key chunk_key(j, r)
         const int key = pc / (HD / 8), part = pc % (HD / 8);
-        *(u32x4*)(stage + key * L::K_STRIDE + part * 16) = rk[i];
+        const int k32 = key & 31;
+        const int krow = (key & 32) + ((k32 >> 2) & 1) * 16 + (k32 >> 3) * 4 + (k32 & 3);
+        *(u32x4*)(stage + krow * L::K_STRIDE + part * 16) = rk[i];
         const int d = pc >> 3, vpart = pc & 7;
         u32x4 v = rv[i];
         if (tail) {
@@ -409,14 +408,7 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_rows_kernel
         }
 #pragma unroll
         for (int dt = 0; dt < HD / 16; ++dt) {
-          const unsigned char* vr = cur + L::K_BYTES + (dt * 16 + c16) * L::V_STRIDE + half * 64 + g * 8;
-          const u32x2 v0 = *(const u32x2*)vr;
-          const u32x2 v1 = *(const u32x2*)(vr + 32);
-          u32x4 vv;
-          vv[0] = v0[0];
-          vv[1] = v0[1];
-          vv[2] = v1[0];
-          vv[3] = v1[1];
+          const u32x4 vv = *(const u32x4*)(cur + L::K_BYTES + (dt * 16 + c16) * L::V_STRIDE + half * 64 + g * 16);
           w.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vv), pb, w.o[qt][dt], 0, 0, 0);
         }
       }
@@ -645,14 +637,26 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
   const int per_wave = (HD * G + 2 * G) * (int)sizeof(float);
   const int fit = (48 * 1024) / per_wave;
   dim3 grid(a.batch, a.nkv, a.nsplit);
-  if (fit >= 16 && HD <= 64) {
-    attn_heads_kernel<HD, 16><<<grid, 16 * 64, (size_t)16 * per_wave, stream>>>(a);
-  } else if (fit >= 8) {
-    attn_heads_kernel<HD, 8><<<grid, 8 * 64, (size_t)8 * per_wave, stream>>>(a);
-  } else if (fit >= 4) {
-    attn_heads_kernel<HD, 4><<<grid, 4 * 64, (size_t)4 * per_wave, stream>>>(a);
-  } else {
-    attn_heads_kernel<HD, 2><<<grid, 2 * 64, (size_t)2 * per_wave, stream>>>(a);
+  // (head sizes above 128 keep to 4 waves: a block of 256 threads may use the whole register file, and
+  // these sizes need more than half of it for one chunk in flight and one being multiplied)
+  bool launched = false;
+  if constexpr (HD <= 64) {
+    if (fit >= 16) {
+      attn_heads_kernel<HD, 16><<<grid, 16 * 64, (size_t)16 * per_wave, stream>>>(a);
+      launched = true;
+    }
+  }
+  if constexpr (HD <= 128) {
+    if (!launched && fit >= 8) {
+      attn_heads_kernel<HD, 8><<<grid, 8 * 64, (size_t)8 * per_wave, stream>>>(a);
+      launched = true;
+    }
+  }
+  if (!launched) {
+    if (fit >= 4)
+      attn_heads_kernel<HD, 4><<<grid, 4 * 64, (size_t)4 * per_wave, stream>>>(a);
+    else
+      attn_heads_kernel<HD, 2><<<grid, 2 * 64, (size_t)2 * per_wave, stream>>>(a);
   }
   LQ_CHECK_LAUNCH("attention(mfma heads)");
   if (a.nsplit > 1) {
