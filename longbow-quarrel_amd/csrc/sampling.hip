@@ -48,6 +48,13 @@ __device__ inline unsigned long long shfl_xor_u64(unsigned long long v, int off)
   return ((unsigned long long)hi << 32) | lo;
 }
 
+__device__ inline unsigned long long shfl_up_u64(unsigned long long v, int off) {
+  unsigned lo = (unsigned)v, hi = (unsigned)(v >> 32);
+  lo = __shfl_up(lo, off, 64);
+  hi = __shfl_up(hi, off, 64);
+  return ((unsigned long long)hi << 32) | lo;
+}
+
 __device__ inline double shfl_f64(double v, int src) {
   const unsigned long long bits = (unsigned long long)__double_as_longlong(v);
   const unsigned hi = __shfl((unsigned)(bits >> 32), src, 64), lo = __shfl((unsigned)bits, src, 64);
@@ -428,9 +435,11 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a) {
     }
     if (select) {
       const float d = (mx - v) * inv_width;
-      const int bin = (d >= 0.f && d < (float)(HIST_BINS - 1)) ? (int)d : HIST_BINS - 1;  // NaN: the last bin
-      atomicAdd(&hist_count[bin], 1u);
-      atomicAdd(&hist_mass[bin], (unsigned long long)((double)e * MASS_UNIT));
+      if (d >= 0.f && d < (float)(HIST_BINS - 1)) {  // beyond: no candidate (and NaN); the cut never looks there
+        const int bin = (int)d;
+        atomicAdd(&hist_count[bin], 1u);
+        atomicAdd(&hist_mass[bin], (unsigned long long)((double)e * MASS_UNIT));
+      }
     }
   });
   const long long ncand = block_sum_i64(ncand_loc, smu);
@@ -441,28 +450,49 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a) {
   // A cut in the histogram: the first bins that surely hold more than the kept set (more than top_k
   // keys, or a mass past top_p by a margin and then one more non-empty bin).  The keys of these bins
   // become a short list in LDS, on which the threshold is then found exactly.
-  if (tid == 0) {
+  if (wave == 0) {
     int cut = -1;
     if (select) {
-      unsigned long long cum_n = 0ull, cum_m = 0ull;
+      // lane l owns bins [16 l, 16 l + 16); running totals up to its first bin by a wave scan
+      constexpr int PER = HIST_BINS / 64;
       const unsigned long long m_need = (unsigned long long)(p_mass * (1.0 + 1e-9) * MASS_UNIT) + (unsigned long long)V + 1ull;
-      bool mass_passed = false;
-      for (int bin = 0; bin < HIST_BINS - 1; ++bin) {
-        const unsigned n_here = hist_count[bin];
-        if (mass_passed && n_here > 0u) {
-          cut = bin;
-          break;
-        }
-        cum_n += n_here;
-        cum_m += hist_mass[bin];
-        if (a.top_k > 0 && cum_n > (unsigned long long)a.top_k) {
-          cut = bin;
-          break;
-        }
-        if (use_p && cum_m >= m_need) mass_passed = true;
+      unsigned long long n_mine = 0ull, m_mine = 0ull;
+      for (int j = 0; j < PER; ++j) {
+        n_mine += hist_count[lane * PER + j];
+        m_mine += hist_mass[lane * PER + j];
       }
+      unsigned long long n_incl = n_mine, m_incl = m_mine;
+      for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long on = shfl_up_u64(n_incl, off), om = shfl_up_u64(m_incl, off);
+        if (lane >= off) {
+          n_incl += on;
+          m_incl += om;
+        }
+      }
+      unsigned long long cum_n = n_incl - n_mine, cum_m = m_incl - m_mine;
+      int bin_k = HIST_BINS, bin_m = HIST_BINS;  // the first bin after which more than top_k keys / the mass are in
+      for (int j = 0; j < PER; ++j) {
+        const int bin = lane * PER + j;
+        cum_n += hist_count[bin];
+        cum_m += hist_mass[bin];
+        if (a.top_k > 0 && cum_n > (unsigned long long)a.top_k && bin_k == HIST_BINS) bin_k = bin;
+        if (use_p && cum_m >= m_need && bin_m == HIST_BINS) bin_m = bin;
+      }
+      for (int off = 32; off > 0; off >>= 1) {
+        bin_k = min(bin_k, __shfl_xor(bin_k, off, 64));
+        bin_m = min(bin_m, __shfl_xor(bin_m, off, 64));
+      }
+      // past the mass: one more non-empty bin
+      int after = HIST_BINS;
+      for (int j = PER - 1; j >= 0; --j) {
+        const int bin = lane * PER + j;
+        if (bin > bin_m && hist_count[bin] > 0u) after = bin;
+      }
+      for (int off = 32; off > 0; off >>= 1) after = min(after, __shfl_xor(after, off, 64));
+      const int first = min(bin_k, after);
+      if (first < HIST_BINS - 1) cut = first;
     }
-    cut_bin = cut;
+    if (lane == 0) cut_bin = cut;
   }
   __syncthreads();
   const int cut = cut_bin;
