@@ -60,6 +60,24 @@ __device__ inline unsigned pack_bf16(float lo, float hi) {
   return c.u;
 }
 
+// Reductions over the four 16-lane rows of a wave (the lanes that share lane % 16) with the row-swap
+// instructions of gfx950, which stay in the vector unit (a shuffle goes through LDS and back).
+// v_permlane16_swap exchanges the odd rows of its first operand with the even rows of its second;
+// with the same value in both, every lane then holds its own and its xor-16 partner's value, the
+// lower row's first.  v_permlane32_swap does the same with the wave's halves.
+__device__ inline float rows_max(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ inline float rows_sum(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // 2^x for x <= 0 (v_exp_f32; results below the normal range flush to zero, which is what a
 // probability that small is worth)
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -93,8 +111,7 @@ __device__ inline float softmax_chunk(const f32x4 (&s)[2], float c, bool masked,
       }
   }
   float cmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-  cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
-  cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+  cmax = rows_max(cmax);
   const float m_new = fmaxf(m, cmax * c);  // c > 0: scaling commutes with the maximum
   const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a column with no key yet
   const float alpha = fast_exp2(m - m_safe);
@@ -426,8 +443,7 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_r
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     float l = w.l[qt];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    l = rows_sum(l);
     if (!w.valid[qt]) continue;
     const float inv = 1.0f / l;
     bf16_t* orow = a.out + (long long)(r0 + qt * 16 + c16) * a.ldo + h * HD + g * 4;
@@ -547,8 +563,7 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
   while (t_first < s_begin) t_first += NW * 32;
   attend<HD, 1>(a, w, kvh, table, t_first, NW * 32, s_end, p);
   float l = w.l[0];
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
+  l = rows_sum(l);
 
   // combine the waves' partial results in wave order
   if (c16 < G) {
