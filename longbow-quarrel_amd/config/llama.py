@@ -6,7 +6,7 @@ count required :465-469, feed-forward width :473-478, kv heads default to heads
 :482-506, head size = width / heads :509-511, context :515-519, rope base 10000
 :523-530, eps 1e-5 :536-542) and its checks (internal/config/config.go:57-105;
 heads % kv_heads in internal/engine/validation.go:52-54), with config.json's key
-names in place of the GGUF ones.  `rope_scaling` (type `llama3`) has no
+names in place of the GGUF ones.  `rope_scaling` (types `llama3` and `linear`; `default` means none) has no
 counterpart in the reference.
 """
 from __future__ import annotations
@@ -20,51 +20,54 @@ from .base import ConfigError, ModelConfig, coerce, optional, require
 
 @dataclass(frozen=True)
 class RopeScaling:
-    """`rope_scaling` of type `llama3`: low frequencies divided by `factor`,
-    high ones kept, a linear blend between the two thresholds."""
+    """`rope_scaling` of type `llama3` (low frequencies divided by `factor`, high ones kept, a
+    linear blend between the two thresholds) or `linear` (every frequency divided by `factor`;
+    the other fields are None)."""
 
     rope_type: str
     factor: float
-    low_freq_factor: float
-    high_freq_factor: float
-    original_max_position_embeddings: int
+    low_freq_factor: Optional[float] = None
+    high_freq_factor: Optional[float] = None
+    original_max_position_embeddings: Optional[int] = None
 
     @classmethod
-    def from_dict(cls, d: Dict[str, Any]) -> "RopeScaling":
+    def from_dict(cls, d: Dict[str, Any]) -> Optional["RopeScaling"]:
+        """None for the type `default` (frequencies as they are)."""
         if not isinstance(d, dict):
             raise ConfigError(f"config.json: 'rope_scaling' must be an object, found {d!r}")
         kind = d.get("rope_type", d.get("type"))
         if kind is None:
             raise ConfigError("config.json: 'rope_scaling' has neither 'rope_type' nor 'type'")
-        if kind != "llama3":
+        if kind == "default":
+            return None
+        if kind not in ("llama3", "linear"):
             raise ConfigError(
-                f"config.json: rope_scaling type {kind!r} is not supported (supported: 'llama3')"
+                f"config.json: rope_scaling type {kind!r} is not supported (supported: 'default', 'linear', 'llama3')"
             )
+        keys = [("factor", float)]
+        if kind == "llama3":
+            keys += [("low_freq_factor", float), ("high_freq_factor", float), ("original_max_position_embeddings", int)]
         vals = {}
-        for key, typ in (
-            ("factor", float),
-            ("low_freq_factor", float),
-            ("high_freq_factor", float),
-            ("original_max_position_embeddings", int),
-        ):
+        for key, typ in keys:
             if key not in d or d[key] is None:
                 raise ConfigError(f"config.json: rope_scaling.{key} is missing")
             vals[key] = coerce(d[key], "rope_scaling." + key, typ)
         if vals["factor"] < 1.0:
             raise ConfigError(f"config.json: rope_scaling.factor must be >= 1, found {vals['factor']}")
-        if not vals["high_freq_factor"] > vals["low_freq_factor"]:
-            raise ConfigError(
-                "config.json: rope_scaling.high_freq_factor must exceed low_freq_factor "
-                f"(found {vals['high_freq_factor']} and {vals['low_freq_factor']})"
-            )
-        if vals["low_freq_factor"] <= 0:
-            raise ConfigError("config.json: rope_scaling.low_freq_factor must be positive")
-        if vals["original_max_position_embeddings"] <= 0:
-            raise ConfigError("config.json: rope_scaling.original_max_position_embeddings must be positive")
-        return cls(rope_type="llama3", **vals)
+        if kind == "llama3":
+            if not vals["high_freq_factor"] > vals["low_freq_factor"]:
+                raise ConfigError(
+                    "config.json: rope_scaling.high_freq_factor must exceed low_freq_factor "
+                    f"(found {vals['high_freq_factor']} and {vals['low_freq_factor']})"
+                )
+            if vals["low_freq_factor"] <= 0:
+                raise ConfigError("config.json: rope_scaling.low_freq_factor must be positive")
+            if vals["original_max_position_embeddings"] <= 0:
+                raise ConfigError("config.json: rope_scaling.original_max_position_embeddings must be positive")
+        return cls(rope_type=kind, **vals)
 
     def to_dict(self) -> Dict[str, Any]:
-        return dataclasses.asdict(self)
+        return {k: v for k, v in dataclasses.asdict(self).items() if v is not None}
 
 
 @dataclass(frozen=True)
@@ -114,7 +117,16 @@ class LlamaConfig(ModelConfig):
         else:
             eos_ids = (coerce(eos, "eos_token_id", int),)
         bos = d.get("bos_token_id")
+        # newer config files keep the base and the scaling together under `rope_parameters`
+        rope = d.get("rope_parameters") if isinstance(d.get("rope_parameters"), dict) else {}
         scaling = d.get("rope_scaling")
+        if scaling is None and rope.get("rope_type", rope.get("type")) is not None:
+            scaling = rope
+        theta = d["rope_theta"] if d.get("rope_theta") is not None else rope.get("rope_theta", 10000.0)
+        act = d.get("hidden_act", "silu")
+        if act not in ("silu", "swish"):
+            # the feed-forward is silu(gate) * up: internal/device/cpu_ref.go:132-149
+            raise ConfigError(f"config.json: 'hidden_act' {act!r} is not supported (supported: 'silu')")
         for key in ("attention_bias", "mlp_bias"):
             if d.get(key):
                 # the reference accepts no bias tensor: internal/engine/engine.go:416-425
@@ -129,7 +141,7 @@ class LlamaConfig(ModelConfig):
             vocab_size=vocab,
             max_position_embeddings=optional(d, "max_position_embeddings", 2048),
             rms_norm_eps=optional(d, "rms_norm_eps", 1e-5, float),
-            rope_theta=optional(d, "rope_theta", 10000.0, float),
+            rope_theta=coerce(theta, "rope_theta", float),
             rope_scaling=RopeScaling.from_dict(scaling) if scaling is not None else None,
             tie_word_embeddings=optional(d, "tie_word_embeddings", False, bool),
             bos_token_id=None if bos is None else coerce(bos, "bos_token_id", int),

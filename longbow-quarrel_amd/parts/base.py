@@ -82,7 +82,7 @@ class TensorSpec:
     name: str  # the safetensors name
     shape: Tuple[int, ...]
     kind: str = MATRIX
-    init: str = "normal"  # random-weights rule: "normal" | "ones" | "zeros"
+    init: str = "normal"  # random-weights rule: "normal" | "around_one" (a gain) | "zeros"
     optional: bool = False  # may be absent from the file (a tied head)
 
 

@@ -23,7 +23,7 @@ class RMSNorm(Norm):
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.name, (self.width,), kind=VECTOR32, init="ones")]
+        return [TensorSpec(self.name, (self.width,), kind=VECTOR32, init="around_one")]
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         super().bind(tensors, env)

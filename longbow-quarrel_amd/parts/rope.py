@@ -2,10 +2,11 @@
 
 f_i = base^(-2 i / hd), angle = position * f_i
 (internal/device/kernels.metal:430-463, host twin internal/device/cpu_ref.go:103-129).
-The optional `llama3` scaling of the frequencies has no counterpart in the
-reference: with wavelength L_i = 2 pi / f_i, L_i < original / high_freq_factor
-keeps f_i, L_i > original / low_freq_factor gives f_i / factor, and between the
-two s = (original / L_i - low) / (high - low), f_i' = (1 - s) f_i / factor + s f_i.
+The optional scaling of the frequencies has no counterpart in the reference.
+`linear` divides every f_i by the factor.  `llama3`: with wavelength
+L_i = 2 pi / f_i, L_i < original / high_freq_factor keeps f_i,
+L_i > original / low_freq_factor gives f_i / factor, and between the two
+s = (original / L_i - low) / (high - low), f_i' = (1 - s) f_i / factor + s f_i.
 
 The table is computed once in float64 and handed to the kernel as a parameter,
 so the kernel knows nothing about scaling types.
@@ -25,6 +26,11 @@ def rotary_frequencies(head_dim: int, base: float, scaling: Optional[Mapping] = 
     if not scaling:
         return freqs
     factor = float(scaling["factor"])
+    kind = scaling.get("rope_type", "llama3")
+    if kind == "linear":  # positions divided by the factor
+        return [f / factor for f in freqs]
+    if kind != "llama3":
+        raise ValueError(f"rope scaling type {kind!r} is not known (known: 'linear', 'llama3')")
     low = float(scaling["low_freq_factor"])
     high = float(scaling["high_freq_factor"])
     original = float(scaling["original_max_position_embeddings"])

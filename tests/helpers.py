@@ -40,7 +40,7 @@ TINY_C = {
 def write_folder(tmp_path, cfg: Dict, seed: int, dtype=None, std: float = 0.02) -> str:
     config = lq.LlamaConfig.from_dict(cfg)
     folder = os.path.join(str(tmp_path), f"model_{seed}_{cfg['hidden_size']}")
-    lq.write_model_folder(folder, config, seed, dtype=dtype, std=std)
+    lq.write_model_folder(folder, config, seed, dtype=dtype, std=std, gain_spread=0.3)
     return folder
 
 

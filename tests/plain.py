@@ -183,7 +183,9 @@ class PlainLlama:
         self.eps = c.get("rms_norm_eps", 1e-5)
         freqs = rope_frequencies(self.hd, c.get("rope_theta", 10000.0))
         rs = c.get("rope_scaling")
-        if rs:
+        if rs and rs.get("rope_type", rs.get("type")) == "linear":
+            freqs = freqs / rs["factor"]  # positions divided by the factor
+        elif rs and rs.get("rope_type", rs.get("type")) != "default":
             freqs = llama3_scaled_frequencies(
                 freqs,
                 rs["factor"],

@@ -53,6 +53,24 @@ def test_config_defaults_follow_the_reference():
     assert c.rope_scaling is None and not c.tie_word_embeddings and c.eos_token_ids == ()
 
 
+def test_other_ways_to_write_the_rotation():
+    d = dict(TINY_A)
+    d["rope_scaling"] = {"rope_type": "default"}
+    assert LlamaConfig.from_dict(d).rope_scaling is None
+    d["rope_scaling"] = {"type": "linear", "factor": 4}
+    c = LlamaConfig.from_dict(d)
+    assert c.rope_scaling.rope_type == "linear" and c.rope_scaling.factor == 4.0
+    assert c.to_dict()["rope_scaling"] == {"rope_type": "linear", "factor": 4.0}
+    assert LlamaConfig.from_dict(c.to_dict()) == c
+    # base and scaling together under `rope_parameters`
+    d = {k: v for k, v in TINY_B.items() if k not in ("rope_scaling", "rope_theta")}
+    d["rope_parameters"] = dict(TINY_B["rope_scaling"], rope_theta=TINY_B["rope_theta"])
+    assert LlamaConfig.from_dict(d) == LlamaConfig.from_dict(TINY_B)
+    d["rope_parameters"] = {"rope_type": "default", "rope_theta": 1234.0}
+    c = LlamaConfig.from_dict(d)
+    assert c.rope_scaling is None and c.rope_theta == 1234.0
+
+
 @pytest.mark.parametrize("change,needle", [
     ({"num_attention_heads": None}, "num_attention_heads"),
     ({"intermediate_size": None}, "intermediate_size"),
@@ -73,6 +91,8 @@ def test_config_defaults_follow_the_reference():
     ({"rope_scaling": {"rope_type": "llama3", "factor": 0.5, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
                        "original_max_position_embeddings": 64}}, "factor"),
     ({"torch_dtype": "int8"}, "torch_dtype"),
+    ({"hidden_act": "gelu"}, "hidden_act"),
+    ({"rope_scaling": {"rope_type": "linear"}}, "factor"),
 ])
 def test_config_errors_name_the_key(change, needle):
     d = dict(TINY_A)
@@ -234,7 +254,8 @@ def test_random_weights_depend_on_seed_and_name_only(tmp_path):
     c = read_folder(write_folder(tmp_path / "z", TINY_A, 8))[1]
     assert all(torch.equal(a[n], b[n]) for n in a)
     assert not torch.equal(a["model.embed_tokens.weight"], c["model.embed_tokens.weight"])
-    assert torch.equal(a["model.norm.weight"], torch.ones(64))
+    gain = a["model.norm.weight"].float()  # around one, and not one: a gain that is left out must show
+    assert abs(float(gain.mean()) - 1.0) < 0.2 and float(gain.std()) > 0.1
     w = a["model.layers.0.mlp.gate_proj.weight"]
     assert abs(float(w.std()) - 0.02) < 0.002 and abs(float(w.mean())) < 0.002
     assert not torch.equal(w, a["model.layers.1.mlp.gate_proj.weight"])

@@ -72,11 +72,13 @@ def test_rotary_encoding_alone_with_and_without_scaling(kn, dtype):
     env = BuildEnv(dtype, DEV, kn)
     scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
                "original_max_position_embeddings": 64}
-    for sc in (None, scaling):
+    for sc in (None, scaling, {"rope_type": "linear", "factor": 4.0}):
         pos = build_part(POSITION_ENCODINGS, PartSpec("rope", {"head_dim": 32, "base": 500000.0, "scaling": sc}))
         pos.bind({}, env)
         want_f = plain.rope_frequencies(32, 500000.0)
-        if sc:
+        if sc and sc["rope_type"] == "linear":
+            want_f = want_f / 4.0
+        elif sc:
             want_f = plain.llama3_scaled_frequencies(want_f, 8.0, 1.0, 4.0, 64)
         assert torch.allclose(pos.rotary_frequencies.cpu(), want_f, rtol=1e-14, atol=0)
         ctx = context(kn, dtype, [300, 7], [4, 2], [1, 0])
