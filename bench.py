@@ -34,6 +34,15 @@ CONFIG_8B = {
 }
 
 
+# the other two shapes that the reference's model family names; the default run and the driver use the 8B one
+CONFIG_1B = dict(CONFIG_8B, hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, head_dim=64,
+                 max_position_embeddings=8192, tie_word_embeddings=True,
+                 rope_scaling={"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                               "original_max_position_embeddings": 8192})
+CONFIG_70B = dict(CONFIG_8B, hidden_size=8192, intermediate_size=28672, num_hidden_layers=80, num_attention_heads=64)
+SHAPES = {"8b": CONFIG_8B, "1b": CONFIG_1B, "70b": CONFIG_70B}
+
+
 def weight_bytes_per_step(c) -> float:
     """Every weight a decode step uses, once: the layers' matrices and norms, the final norm and the head
     (of the embedding table only the batch's rows are read)."""
@@ -63,6 +72,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the 8B shape has (0 = all 32)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--prompt-len-max", type=int, default=0,
+                    help="prompts of unequal lengths, uniform in [--prompt-len, this] (0 = all of --prompt-len)")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (the headline run is 8b)")
     ap.add_argument("--no-points", action="store_true", help="skip the prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
     args = ap.parse_args()
@@ -75,7 +87,7 @@ def main() -> int:
     import longbow_quarrel_amd as lq
     from longbow_quarrel_amd.engine import EngineBackend, StepEntry
 
-    cfg = dict(CONFIG_8B)
+    cfg = dict(SHAPES[args.shape])
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -95,10 +107,13 @@ def main() -> int:
         """tokens a second, ms a step, mean context during the timed steps"""
         backend = EngineBackend(engine, lq.SamplingParams(temperature=0.0), use_graphs=True)
         slots = [backend.new_sequence(r, [0]) for r in range(batch)]
-        prompts = [random_prompt(prompt_len) for _ in range(batch)]
+        lens = [prompt_len] * batch
+        if args.prompt_len_max > prompt_len:
+            lens = torch.randint(prompt_len, args.prompt_len_max + 1, (batch,), generator=gen).tolist()
+        prompts = [random_prompt(n) for n in lens]
         # prompts in chunks of sequences so that a prefill step stays at a few thousand rows
         toks = []
-        per = max(1, 4096 // prompt_len)
+        per = max(1, 4096 // max(lens))
         for i in range(0, batch, per):
             toks += backend.prefill(slots[i : i + per], prompts[i : i + per])
         for _ in range(warmup):
@@ -109,7 +124,7 @@ def main() -> int:
             toks = backend.decode(slots, toks, False)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
-        ctx_mean = prompt_len + warmup + (steps + 1) / 2.0
+        ctx_mean = sum(lens) / batch + warmup + (steps + 1) / 2.0
         for s in slots:
             backend.release(s)
         backend.close()
@@ -158,12 +173,12 @@ def main() -> int:
         print(f"[bench] points: {points}", file=sys.stderr, flush=True)
 
     line = {
-        "metric": "decode tok/s (Llama-3 8B shape, bf16, batch 8, 512-token prompts)",
+        "metric": f"decode tok/s (Llama-3 {args.shape.upper()} shape, bf16, batch {args.batch}, {args.prompt_len}-token prompts)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic: random weights N(0, 0.02) from a seed, uniform random token ids",
         "config": {
-            "model": "llama3-8b-shape", "layers": config.num_hidden_layers, "layers_full": full_layers,
+            "model": f"llama3-{args.shape}-shape", "layers": config.num_hidden_layers, "layers_full": full_layers,
             "hidden": config.hidden_size, "heads": config.num_attention_heads,
             "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
             "intermediate": config.intermediate_size, "vocab": config.vocab_size,

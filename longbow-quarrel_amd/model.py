@@ -100,10 +100,11 @@ class DecoderModel:
         of the rows listed in want_rows (None when nothing is wanted)."""
         kn = ctx.kernels
         s = self.spec
-        x = ctx.ws.alloc((ctx.rows, s.width), torch.float32)
+        x = ctx.ws.alloc((ctx.rows, s.width), torch.float32, keep=True)
         kn.embed(self.embedding, ctx.tokens, x)
         pending: Optional[torch.Tensor] = None
         for i, run in enumerate(s.schedule):
+            ctx.ws.next_run()  # the buffers of the run before the last one are free again
             cache = caches.get(i if run.cache_of is None else run.cache_of)
             if cache is not None and run.cache_of is not None:
                 cache = LayerCache(write=False, k=cache.k, v=cache.v, block_table=cache.block_table,
@@ -116,6 +117,7 @@ class DecoderModel:
                 pending = block.forward(x, pending, ctx, cache)
         if n_want == 0:
             return None
+        ctx.ws.next_run()
         picked = ctx.ws.alloc((n_want, s.width), torch.float32)
         kn.gather_rows(x, want_rows, picked, delta=None if isinstance(pending, RowStats) else pending)
         normed = self.final_norm.forward(picked, ctx)

@@ -119,31 +119,30 @@ class BuildEnv:
     kernels: Any  # HipKernels, or a test's stand-in with the same methods
 
 
-class Workspace:
-    """Bump allocator over one device buffer; reset at the start of every step.
-
-    Addresses repeat from step to step for equal shapes, which a captured HIP
-    graph relies on.  It grows (outside captures) when a step needs more.
-    """
+class _Arena:
+    """Bump allocator over one device buffer."""
 
     ALIGN = 256
 
-    def __init__(self, device: torch.device, nbytes: int = 1 << 20) -> None:
+    def __init__(self, device: torch.device, nbytes: int) -> None:
         self.device = device
         self.buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
         self.off = 0
         self.high = 0
-        self.frozen = False  # set while a graph that uses this buffer is alive
         self._spill: List[torch.Tensor] = []
 
-    def reset(self) -> None:
-        if self.high > self.buf.numel() and not self.frozen:
+    def rewind(self) -> None:
+        self.off = 0
+        self._spill = []  # (freed in stream order: later kernels of the step may take the memory)
+
+    def reset(self, grow: bool) -> None:
+        if self.high > self.buf.numel() and grow:
             self.buf = torch.empty(int(self.high * 1.25) + self.ALIGN, dtype=torch.uint8, device=self.device)
         self.off = 0
         self.high = 0
         self._spill = []
 
-    def alloc(self, shape, dtype: torch.dtype) -> torch.Tensor:
+    def alloc(self, shape, dtype: torch.dtype, frozen: bool) -> torch.Tensor:
         n = 1
         for s in shape:
             n *= int(s)
@@ -153,12 +152,52 @@ class Workspace:
         self.off = end
         self.high = max(self.high, end)
         if end > self.buf.numel():
-            if self.frozen:
+            if frozen:
                 raise RuntimeError("workspace of a captured graph is too small for this step")
             t = torch.empty(tuple(shape), dtype=dtype, device=self.device)  # this step only; reset() grows
             self._spill.append(t)
             return t
         return self.buf[start:end].view(dtype).view(tuple(shape))
+
+
+class Workspace:
+    """A step's temporary buffers, reset at the start of every step.
+
+    Two lifetimes.  `alloc(..., keep=True)` lasts until the step ends (the residual stream, tables that
+    every layer shares).  A plain `alloc` lasts until the end of the *next* run of the schedule: what a
+    block leaves for the block after it (a pending delta, row statistics) is still there when that block
+    reads it, and the memory is used again two runs later, so a step's footprint is that of two layers,
+    not of all of them.  The model calls `next_run()` before each run of the schedule.
+
+    Addresses repeat from step to step for equal shapes, which a captured HIP
+    graph relies on.  It grows (outside captures) when a step needs more.
+    """
+
+    def __init__(self, device: torch.device, nbytes: int = 1 << 20) -> None:
+        self.device = device
+        self.step = _Arena(device, nbytes)
+        self.runs = [_Arena(device, nbytes), _Arena(device, nbytes)]
+        self.cur = 0
+        self.frozen = False  # set while a graph that uses these buffers is alive
+
+    def reset(self) -> None:
+        for arena in (self.step, *self.runs):
+            arena.reset(grow=not self.frozen)
+        self.cur = 0
+
+    def next_run(self) -> None:
+        """What the run before the last one allocated is given up."""
+        self.cur ^= 1
+        self.runs[self.cur].rewind()
+
+    def alloc(self, shape, dtype: torch.dtype, keep: bool = False) -> torch.Tensor:
+        arena = self.step if keep else self.runs[self.cur]
+        return arena.alloc(shape, dtype, self.frozen)
+
+    @property
+    def high(self) -> int:
+        """Bytes this step has needed so far."""
+        return self.step.high + self.runs[0].high + self.runs[1].high
 
 
 @dataclass

@@ -67,7 +67,7 @@ class RotaryEncoding(PositionEncoding):
         key = ("rope_cos_sin", tuple(self.table))
         table = ctx.shared.get(key)
         if table is None:
-            table = ctx.ws.alloc((ctx.rows, self.head_dim // 2, 2), torch.float32)
+            table = ctx.ws.alloc((ctx.rows, self.head_dim // 2, 2), torch.float32, keep=True)
             ctx.kernels.rope_table(self.rotary_frequencies, ctx.row_pos, table)
             ctx.shared[key] = table
         return table

@@ -131,3 +131,39 @@ def test_toy_parts_register_build_and_step_without_touching_the_framework(tmp_pa
         assert rel_err(eng.step([StepEntry(s, b, range(9))]), wb) < TOL
     finally:
         toy_parts.unregister_toys()
+
+
+def test_workspace_lifetimes():
+    """A plain buffer lasts until the end of the next run of the schedule and its memory comes again two
+    runs later; a kept one lasts the whole step; a step's footprint is that of two runs, however many run."""
+    from longbow_quarrel_amd.parts.base import Workspace
+
+    ws = Workspace(torch.device("cpu"), 1 << 16)
+    ws.reset()
+    kept = ws.alloc((100,), torch.float32, keep=True)
+    kept.fill_(7.0)
+    seen = []
+    for run in range(6):
+        ws.next_run()
+        t = ws.alloc((1000,), torch.float32)
+        t.fill_(float(run))
+        if seen:
+            assert float(seen[-1][0]) == run - 1  # the run before still holds its values
+        seen.append(t)
+    assert seen[0].data_ptr() == seen[2].data_ptr() == seen[4].data_ptr()
+    assert seen[1].data_ptr() == seen[3].data_ptr() != seen[0].data_ptr()
+    assert float(kept[0]) == 7.0 and ws.high < 3 * 4096
+    # a step that outgrows the buffers still runs (from the allocator), and the next step has room
+    ws.next_run()
+    big = ws.alloc((1 << 16,), torch.float32)
+    big.zero_()
+    ws.reset()
+    ws.next_run()
+    again = ws.alloc((1 << 16,), torch.float32)
+    assert again.data_ptr() == ws.runs[ws.cur].buf.data_ptr()
+    # a captured graph's buffers must not move
+    ws.frozen = True
+    ws.reset()
+    ws.next_run()
+    with pytest.raises(RuntimeError, match="too small"):
+        ws.alloc((1 << 20,), torch.float32)
