@@ -8,20 +8,20 @@ int lq_attention_generic(const void* q, int ldq, void* out, int ldo, int dtype, 
                          int window, hipStream_t stream);
 bool lq_attention_mfma_accepts(int dtype, int nh, int nkv, int hd, int block_size, int ldq, int ldo,
                                const void* q, const void* out, int decode);
-long long lq_attention_mfma_workspace(int rows, int nh, int hd, int max_len);
+long long lq_attention_mfma_workspace(int rows, int nh, int nkv, int hd, int max_len);
 int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int batch, int nh, int nkv,
                       int hd, const int* row_pos, const int* seq_slot, const int* cu_rows,
                       const int* block_table, int bt_stride, const void* kcache, const void* vcache,
                       float scale, int window, int decode, int max_len, float* workspace,
-                      long long workspace_floats, const void* k_new, const void* v_new, int ldk, int ldv,
-                      const float* cs, hipStream_t stream);
+                      long long workspace_floats, int* tickets, long long tickets_n, const void* k_new,
+                      const void* v_new, int ldk, int ldv, const float* cs, hipStream_t stream);
 
 // Floats of workspace lq_attention wants for this launch (0: none).
 extern "C" long long lq_attention_workspace(int dtype, int rows, int nh, int nkv, int hd, int block_size,
                                             int decode, int max_len) {
   if (!decode || dtype != LQ_BF16) return 0;
   if (!lq_attention_mfma_accepts(dtype, nh, nkv, hd, block_size, 8, 8, nullptr, nullptr, decode)) return 0;
-  return lq_attention_mfma_workspace(rows, nh, hd, max_len);
+  return lq_attention_mfma_workspace(rows, nh, nkv, hd, max_len);
 }
 
 // Whether a decoding launch can take the rotation of q and k and the cache write upon itself
@@ -31,14 +31,17 @@ extern "C" int lq_attention_folds_rope(int dtype, int nh, int nkv, int hd, int b
 }
 
 // `decode` != 0 promises one row per sequence; `max_len` is then an upper bound of the
-// sequences' lengths after this step (it sizes the split grid, not the result).
+// sequences' lengths after this step (it sizes the split grid, not the result).  `tickets` are
+// counters that are zero between launches (a launch leaves them so): one for each row and kv head.
+// Launches that share them must not overlap.
 extern "C" int lq_attention(const void* q, int ldq, void* out, int ldo, int dtype, int rows, int batch,
                             int nh, int nkv, int hd, const int* row_pos, const int* row_seq,
                             const int* seq_slot, const int* cu_rows, const int* block_table,
                             int bt_stride, const void* kcache, const void* vcache, int block_size,
                             float scale, int window, int decode, int max_len, float* workspace,
-                            long long workspace_floats, const void* k_new, const void* v_new, int ldk, int ldv,
-                            const float* cs, int force_generic, hipStream_t stream) {
+                            long long workspace_floats, int* tickets, long long tickets_n, const void* k_new,
+                            const void* v_new, int ldk, int ldv, const float* cs, int force_generic,
+                            hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && batch > 0, "attention: rows %d and sequences %d must be positive", rows, batch);
   LQ_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "attention: %d heads over %d kv heads", nh, nkv);
   LQ_REQUIRE(hd > 0 && block_size > 0 && bt_stride > 0, "attention: bad sizes");
@@ -49,7 +52,7 @@ extern "C" int lq_attention(const void* q, int ldq, void* out, int ldo, int dtyp
   if (!force_generic && lq_attention_mfma_accepts(dtype, nh, nkv, hd, block_size, ldq, ldo, q, out, decode))
     return lq_attention_mfma(q, ldq, out, ldo, rows, batch, nh, nkv, hd, row_pos, seq_slot, cu_rows,
                              block_table, bt_stride, kcache, vcache, scale, window, decode, max_len,
-                             workspace, workspace_floats, k_new, v_new, ldk, ldv, cs, stream);
+                             workspace, workspace_floats, tickets, tickets_n, k_new, v_new, ldk, ldv, cs, stream);
   LQ_REQUIRE(cs == nullptr, "attention: the folded rotation was asked of a launch the matrix-core kernel does not take");
   return lq_attention_generic(q, ldq, out, ldo, dtype, rows, nh, nkv, hd, row_pos, row_seq, seq_slot,
                               block_table, bt_stride, kcache, vcache, block_size, scale, window, stream);

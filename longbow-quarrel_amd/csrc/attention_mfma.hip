@@ -21,11 +21,15 @@
 //    and reuses every key/value fragment it loads for all of them; the waves of a block are the
 //    query heads of one kv head over the same rows, so that they read the same keys at the same time.
 //  * heads (decoding): one row of one sequence, the query heads of one kv head as the 16 columns.
-//    The waves of a block take the chunks of a split of SPLIT positions in turn (wave w: chunks
-//    w, w + NW, ...) and combine their partial results through LDS in wave order.  A sequence longer
-//    than SPLIT has several blocks, merged by a second kernel in ascending split order.  Splits
-//    and chunks are aligned to absolute positions: the order of every sum depends on the row's
-//    position only.
+//    The waves of a block take the cache blocks (64 positions: two chunks) of a split of
+//    `split_len` positions in turn (wave w: blocks w, w + NW, ...) and combine their partial results
+//    through LDS in wave order.  A compute unit keeps about a hundred memory requests in flight,
+//    whatever their size, so a sequence's keys are spread over many workgroups: a split is 256
+//    positions unless that would make more than MAX_DECODE_BLOCKS workgroups.  A row with several
+//    splits is finished by whichever of its blocks comes last (a ticket counter per row and kv
+//    head), which adds the partial results up in ascending split order: no second kernel, and the
+//    result does not depend on which block that was.  Splits and chunks are aligned to absolute
+//    positions.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -36,7 +40,7 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr int BS = 64;      // positions per cache block (the only block size this file takes)
-constexpr int SPLIT = 1024;  // keys per block when decoding
+constexpr int MAX_DECODE_BLOCKS = 512;  // beyond this, decoding splits grow instead of multiplying
 
 __device__ inline bf16x8 as_bf16x8(u32x4 v) {
   union {
@@ -130,6 +134,18 @@ __device__ inline float softmax_chunk(const f32x4 (&s)[2], float c, bool masked,
   return alpha;
 }
 
+// Partial results that cross from one block of a launch to another.  The L2 caches of the chip's
+// dies are not coherent with each other for ordinary accesses, and the fences that make them so
+// write back and invalidate a whole L2 for everybody.  Device-scope atomic stores and loads go
+// past those caches instead: the writer waits until its stores have completed before it takes its
+// ticket, the reader reads after it has seen the last ticket.
+__device__ inline void publish_result(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline float other_blocks_result(const float* p) {
+  return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 struct AttnArgs {
   const bf16_t* q;
   int ldq;
@@ -150,6 +166,8 @@ struct AttnArgs {
   float* part_o;   // [rows][nh][nsplit][HD]
   float* part_ml;  // [rows][nh][nsplit][2]
   int nsplit;
+  int split_len;   // positions per split, a multiple of 256
+  int* tickets;    // [rows][nkv], zero between launches: how many splits of the row have finished
   // decode with the rotation and the cache write folded in (all null otherwise): the step's
   // unrotated keys and values, and cos/sin of every row's angles [rows][HD/2][2]
   const bf16_t* k_new;
@@ -166,20 +184,29 @@ struct ChunkRegs {
   u32x4 v[HD / 16];
 };
 
-template <int HD>
-__device__ inline void load_chunk(const AttnArgs& a, int kvh, long long blk, int koff, ChunkRegs<HD>& r) {
+// A whole cache block: both chunks of 32 keys.  Every line of the cache is asked for by two
+// instructions next to each other (a key row's k-steps, a value row's two halves), which the L1
+// turns into one request of 128 bytes; halves asked for by different waves go out as two of 64,
+// and it is the number of requests in flight that a compute unit is short of.
+// (Head sizes above 128 have no registers for a whole block: they load chunk by chunk, FIRST to
+// FIRST + N - 1, into r[0 .. N-1].)
+template <int HD, int FIRST, int N>
+__device__ inline void load_block(const AttnArgs& a, int kvh, long long blk, ChunkRegs<HD> (&r)[N]) {
   const int lane = threadIdx.x & 63, c16 = lane & 15, g = lane >> 4;
-  const bf16_t* kb = a.kcache + ((blk * a.nkv + kvh) * BS + koff) * (long long)HD;
+  const bf16_t* kb = a.kcache + ((blk * a.nkv + kvh) * BS) * (long long)HD;
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int hf = 0; hf < N; ++hf)
 #pragma unroll
-    for (int kk = 0; kk < HD / 32; ++kk)
-      r.k[j][kk] = *(const u32x4*)(kb + chunk_key(j, c16) * HD + kk * 32 + g * 8);
-  const bf16_t* vb = a.vcache + ((blk * a.nkv + kvh) * (long long)HD) * BS + koff;
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int kk = 0; kk < HD / 32; ++kk)
+        r[hf].k[j][kk] = *(const u32x4*)(kb + ((FIRST + hf) * 32 + chunk_key(j, c16)) * HD + kk * 32 + g * 8);
+  const bf16_t* vb = a.vcache + ((blk * a.nkv + kvh) * (long long)HD) * BS;
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) {
     const bf16_t* vr = vb + (long long)(dt * 16 + c16) * BS;
-    r.v[dt] = *(const u32x4*)(vr + g * 8);
+#pragma unroll
+    for (int hf = 0; hf < N; ++hf) r[hf].v[dt] = *(const u32x4*)(vr + (FIRST + hf) * 32 + g * 8);
   }
 }
 
@@ -200,61 +227,65 @@ struct QTiles {
   int free_from[QT];  //   visible to every column: no masking needed (wave-uniform; free_to = -1: never)
 };
 
-// Walks chunks t_first, t_first + t_step, ... while <= t_end (all multiples of 32).  Keys beyond
-// t_written were never written and are kept out of the second product.
+// Walks the cache blocks that start at t_first, t_first + t_step, ... while <= t_end (all multiples
+// of 64).  Keys beyond t_written were never written and are kept out of the second product.
 template <int HD, int QT>
 __device__ inline void attend(const AttnArgs& a, QTiles<HD, QT>& w, int kvh, const int* table, int t_first,
                               int t_step, int t_end, int t_written) {
   const int lane = threadIdx.x & 63, g = lane >> 4;
   if (t_first > t_end) return;
-  // the next chunk's keys and values are already on their way while this chunk is computed, and
-  // the block number of the chunk after that while those are loaded
-  ChunkRegs<HD> cur, nxt;
+  // One block a wave is in flight (it fills the compute unit's queue of requests by itself); only
+  // the block number is fetched one round ahead.
+  constexpr int AT_ONCE = HD <= 128 ? 2 : 1;
+  ChunkRegs<HD> blk[AT_ONCE];
   long long blk_next = table[t_first / BS];
-  load_chunk<HD>(a, kvh, blk_next, t_first % BS, nxt);
-  blk_next = (t_first + t_step <= t_end) ? table[(t_first + t_step) / BS] : 0;
-  for (int t0 = t_first; t0 <= t_end; t0 += t_step) {
-    cur = nxt;
-    if (t0 + t_step <= t_end) {
-      load_chunk<HD>(a, kvh, blk_next, (t0 + t_step) % BS, nxt);
-      blk_next = (t0 + 2 * t_step <= t_end) ? table[(t0 + 2 * t_step) / BS] : 0;
-    }
-    // values of keys that were never written must not reach the product (0 * garbage may be NaN)
-    if (t0 + 31 > t_written) {
-      const int ta = t0 + g * 8;  // this lane's eight keys
+  for (int tb = t_first; tb <= t_end; tb += t_step) {
+    const long long blk_now = blk_next;
+    load_block<HD, 0, AT_ONCE>(a, kvh, blk_now, blk);
+    blk_next = (tb + t_step <= t_end) ? table[(tb + t_step) / BS] : 0;
 #pragma unroll
-      for (int dt = 0; dt < HD / 16; ++dt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (ta + 2 * e > t_written) cur.v[dt][e] &= 0xffff0000u;
-          if (ta + 2 * e + 1 > t_written) cur.v[dt][e] &= 0x0000ffffu;
-        }
-    }
-#pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-      if (t0 > w.last_key[qt] || t0 + 31 < w.first_key[qt]) continue;  // nothing of this chunk is visible
-      f32x4 s[2];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        s[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kk = 0; kk < HD / 32; ++kk)
-          s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.k[j][kk]), w.q[qt][kk], s[j], 0, 0, 0);
-      }
-      const bool masked = !(t0 + 31 <= w.free_to[qt] && t0 >= w.free_from[qt]);
-      u32x4 pw;
-      const float alpha = softmax_chunk(s, a.scale_log2, masked, w.valid[qt], t0, w.lo[qt], w.pos[qt], w.m[qt],
-                                        w.l[qt], pw);
-      const bf16x8 pb = as_bf16x8(pw);
-      if (!__all(alpha == 1.0f)) {  // the maximum moved for some column: rescale what has been summed
+    for (int hf = 0; hf < 2; ++hf) {
+      const int t0 = tb + hf * 32;
+      if (t0 > t_end) break;
+      if (AT_ONCE == 1 && hf == 1) load_block<HD, 1, AT_ONCE>(a, kvh, blk_now, blk);
+      ChunkRegs<HD>& cur = blk[AT_ONCE == 2 ? hf : 0];
+      // values of keys that were never written must not reach the product (0 * garbage may be NaN)
+      if (t0 + 31 > t_written) {
+        const int ta = t0 + g * 8;  // this lane's eight keys
 #pragma unroll
         for (int dt = 0; dt < HD / 16; ++dt)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) w.o[qt][dt][e] *= alpha;
+          for (int e = 0; e < 4; ++e) {
+            if (ta + 2 * e > t_written) cur.v[dt][e] &= 0xffff0000u;
+            if (ta + 2 * e + 1 > t_written) cur.v[dt][e] &= 0x0000ffffu;
+          }
       }
 #pragma unroll
-      for (int dt = 0; dt < HD / 16; ++dt)
-        w.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.v[dt]), pb, w.o[qt][dt], 0, 0, 0);
+      for (int qt = 0; qt < QT; ++qt) {
+        if (t0 > w.last_key[qt] || t0 + 31 < w.first_key[qt]) continue;  // nothing of this chunk is visible
+        f32x4 s[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          s[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int kk = 0; kk < HD / 32; ++kk)
+            s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.k[j][kk]), w.q[qt][kk], s[j], 0, 0, 0);
+        }
+        const bool masked = !(t0 + 31 <= w.free_to[qt] && t0 >= w.free_from[qt]);
+        u32x4 pw;
+        const float alpha = softmax_chunk(s, a.scale_log2, masked, w.valid[qt], t0, w.lo[qt], w.pos[qt], w.m[qt],
+                                          w.l[qt], pw);
+        const bf16x8 pb = as_bf16x8(pw);
+        if (!__all(alpha == 1.0f)) {  // the maximum moved for some column: rescale what has been summed
+#pragma unroll
+          for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w.o[qt][dt][e] *= alpha;
+        }
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; ++dt)
+          w.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.v[dt]), pb, w.o[qt][dt], 0, 0, 0);
+      }
     }
   }
 }
@@ -482,7 +513,7 @@ int launch_rows(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
 // Block = NW waves over one split of one (sequence, kv head).  LDS: per wave HD x G floats of
 // partial output (the valid columns only), G maxima, G normalisers.
 template <int HD, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
+__global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int G = a.nh / a.nkv;
   float* lds_o = lds;                    // [NW][HD][G]
@@ -491,33 +522,40 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
   const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, g = lane >> 4;
   const int r = b;  // a decoding step has one row a sequence, in the order of the sequences
+  // Everything that depends on the row alone is asked for at once, before the position is known:
+  // a block's time is a chain of memory round trips (position, block table, keys), and these join
+  // the first of them.
   const int p = a.row_pos[r];
-  const int lo = (a.window > 0 && p >= a.window) ? p - a.window + 1 : 0;
-  const int s_begin = max(split * SPLIT, (lo / 32) * 32);
-  const int s_end = min(split * SPLIT + SPLIT - 1, p);
-  if (s_begin > s_end) return;  // the whole block: this split holds no key of the row
-  const int* table = a.block_table + (long long)a.seq_slot[b] * a.bt_stride;
+  const int slot = a.seq_slot[b];
   const int h = kvh * G + min(c16, G - 1);
-
-  QTiles<HD, 1> w;
-  init_tiles<HD, 1>(w);
-  w.valid[0] = c16 < G;
-  w.pos[0] = p;
-  w.lo[0] = lo;
-  w.last_key[0] = p;
-  w.first_key[0] = lo;
-  w.free_to[0] = -1;  // columns beyond the group's heads are never valid: always the masked path
-  w.free_from[0] = 0;
+  const bool folded = HD % 64 == 0 && a.cs != nullptr;
   u32x4 qraw[HD / 32];
   {
     const bf16_t* qr = a.q + (long long)r * a.ldq + h * HD + g * 8;
 #pragma unroll
     for (int kk = 0; kk < HD / 32; ++kk) qraw[kk] = *(const u32x4*)(qr + kk * 32);
   }
-  if (HD % 64 == 0 && a.cs != nullptr) {
-    // The rotation and the cache write of this step, folded in.  Pair (i, i + HD/2): a lane's
-    // fragment kk holds i = kk*32 + (lane/16)*8 + j and its fragment kk + HD/64 the partners.
+  // the row's own key and value (lane i: pair i of the key, elements d of the value), for the wave
+  // that will turn out to write them
+  constexpr int KP = (HD / 2 + 63) / 64, VP = (HD + 63) / 64;
+  float kx0[KP], kx1[KP], kc[KP], ks[KP];
+  bf16_t vx[VP];
+  if (folded) {
     const float* cs = a.cs + (long long)r * HD;  // [HD/2][2]
+    const bf16_t* kr = a.k_new + (long long)r * a.ldk + kvh * HD;
+    const bf16_t* vr = a.v_new + (long long)r * a.ldv + kvh * HD;
+#pragma unroll
+    for (int j = 0; j < KP; ++j) {
+      const int i = min(lane + 64 * j, HD / 2 - 1);
+      kx0[j] = bf16_to_f32(kr[i]);
+      kx1[j] = bf16_to_f32(kr[i + HD / 2]);
+      kc[j] = cs[2 * i];
+      ks[j] = cs[2 * i + 1];
+    }
+#pragma unroll
+    for (int j = 0; j < VP; ++j) vx[j] = vr[min(lane + 64 * j, HD - 1)];
+    // The rotation of this step's query, folded in.  Pair (i, i + HD/2): a lane's
+    // fragment kk holds i = kk*32 + (lane/16)*8 + j and its fragment kk + HD/64 the partners.
 #pragma unroll
     for (int kk = 0; kk < HD / 64; ++kk) {
       const int i0 = kk * 32 + g * 8;
@@ -533,35 +571,62 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
       qraw[kk] = lo4;
       qraw[kk + HD / 64] = hi4;
     }
-    // The wave that will read the chunk holding position p writes the row's rotated key and its
-    // value there first; a workgroup-scope fence orders its lanes' stores before its lanes' loads.
-    // No other wave (and no other block) reads that chunk.
-    if (split == p / SPLIT && wave == ((p - split * SPLIT) / 32) % NW) {
-      const long long blk = table[p / BS];
-      const int off = p % BS;
-      const bf16_t* kr = a.k_new + (long long)r * a.ldk + kvh * HD;
-      const bf16_t* vr = a.v_new + (long long)r * a.ldv + kvh * HD;
-      bf16_t* kdst = const_cast<bf16_t*>(a.kcache) + ((blk * a.nkv + kvh) * BS + off) * (long long)HD;
-      bf16_t* vdst = const_cast<bf16_t*>(a.vcache) + ((blk * a.nkv + kvh) * (long long)HD) * BS + off;
-      for (int i = lane; i < HD / 2; i += 64) {
-        const float x0 = bf16_to_f32(kr[i]), x1 = bf16_to_f32(kr[i + HD / 2]);
-        const float c = cs[2 * i], sn = cs[2 * i + 1];
+#pragma unroll
+    for (int j = 0; j < KP; ++j) {  // the key's rotation, by every wave: whoever writes it has it ready
+      const float x0 = kx0[j], x1 = kx1[j];
+      kx0[j] = x0 * kc[j] - x1 * ks[j];
+      kx1[j] = x0 * ks[j] + x1 * kc[j];
+    }
+  }
+  const int lo = (a.window > 0 && p >= a.window) ? p - a.window + 1 : 0;
+  const int SL = a.split_len, lo64 = (lo / BS) * BS;
+  const int s_begin = max(split * SL, lo64);
+  const int s_end = min(split * SL + SL - 1, p);
+  if (s_begin > s_end) return;  // the whole block: this split holds no key of the row
+  const int s_first = lo64 / SL, s_last = p / SL;  // the row's splits that hold keys
+  const int* table = a.block_table + (long long)slot * a.bt_stride;
+
+  QTiles<HD, 1> w;
+  init_tiles<HD, 1>(w);
+  w.valid[0] = c16 < G;
+  w.pos[0] = p;
+  w.lo[0] = lo;
+  w.last_key[0] = p;
+  w.first_key[0] = lo;
+  w.free_to[0] = -1;  // columns beyond the group's heads are never valid: always the masked path
+  w.free_from[0] = 0;
+  // The wave that will read the block holding position p writes the row's rotated key and its
+  // value there first; a workgroup-scope fence orders its lanes' stores before its lanes' loads.
+  // No other wave (and no other workgroup) reads that block.
+  if (folded && split == s_last && wave == ((p - split * SL) / BS) % NW) {
+    const long long blk = table[p / BS];
+    const int off = p % BS;
+    bf16_t* kdst = const_cast<bf16_t*>(a.kcache) + ((blk * a.nkv + kvh) * BS + off) * (long long)HD;
+    bf16_t* vdst = const_cast<bf16_t*>(a.vcache) + ((blk * a.nkv + kvh) * (long long)HD) * BS + off;
+#pragma unroll
+    for (int j = 0; j < KP; ++j) {
+      const int i = lane + 64 * j;
+      if (i < HD / 2) {
         bf16_t r0, r1;
-        r0.bits = (uint16_t)(pack_bf16(x0 * c - x1 * sn, 0.f) & 0xffffu);
-        r1.bits = (uint16_t)(pack_bf16(x0 * sn + x1 * c, 0.f) & 0xffffu);
+        r0.bits = (uint16_t)(pack_bf16(kx0[j], 0.f) & 0xffffu);
+        r1.bits = (uint16_t)(pack_bf16(kx1[j], 0.f) & 0xffffu);
         kdst[i] = r0;
         kdst[i + HD / 2] = r1;
       }
-      for (int d = lane; d < HD; d += 64) vdst[(long long)d * BS] = vr[d];
-      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
     }
+#pragma unroll
+    for (int j = 0; j < VP; ++j) {
+      const int d = lane + 64 * j;
+      if (d < HD) vdst[(long long)d * BS] = vx[j];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
   }
 #pragma unroll
   for (int kk = 0; kk < HD / 32; ++kk) w.q[0][kk] = as_bf16x8(qraw[kk]);
-  // chunk numbering is absolute within the split, so that a wave's chunks depend on positions only
-  int t_first = split * SPLIT + wave * 32;
-  while (t_first < s_begin) t_first += NW * 32;
-  attend<HD, 1>(a, w, kvh, table, t_first, NW * 32, s_end, p);
+  // block numbering is absolute within the split, so that a wave's blocks depend on positions only
+  int t_first = split * SL + wave * BS;
+  while (t_first < s_begin) t_first += NW * BS;
+  attend<HD, 1>(a, w, kvh, table, t_first, NW * BS, s_end, p);
   float l = w.l[0];
   l = rows_sum(l);
 
@@ -593,50 +658,61 @@ __global__ __launch_bounds__(NW * 64) void attn_heads_kernel(AttnArgs a) {
       L += wgt * lds_l[j * G + c];
     }
     const int hh = kvh * G + c;
-    if (a.nsplit == 1) {
+    if (s_first == s_last) {
       a.out[(long long)r * a.ldo + hh * HD + d] = f32_to_bf16(acc / L);
     } else {
       const long long slot = ((long long)r * a.nh + hh) * a.nsplit + split;
-      a.part_o[slot * HD + d] = acc;
+      publish_result(a.part_o + slot * HD + d, acc);
       if (d == 0) {
-        a.part_ml[slot * 2] = M;
-        a.part_ml[slot * 2 + 1] = L;
+        publish_result(a.part_ml + slot * 2, M);
+        publish_result(a.part_ml + slot * 2 + 1, L);
       }
     }
   }
-}
+  if (s_first == s_last) return;
 
-// Merges the splits of one (row, head): out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s,
-// splits in ascending order.
-template <int HD>
-__global__ __launch_bounds__(64) void attn_merge_kernel(AttnArgs a) {
-  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int r = b;
-  const int p = a.row_pos[r];
-  const int lo = (a.window > 0 && p >= a.window) ? p - a.window + 1 : 0;
-  const int s_first = lo / SPLIT, s_last = p / SPLIT;
-  const long long base = ((long long)r * a.nh + h) * a.nsplit;
-  float M = -INFINITY;
-  for (int s = s_first; s <= s_last; ++s) M = fmaxf(M, a.part_ml[(base + s) * 2]);
-  float L = 0.f;
-  float acc[HD / 64 + 1];
+  // The row has other splits.  Once every thread's stores have completed the block takes a ticket;
+  // the block that takes the last one adds the splits up.
+  __shared__ int last_block;
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's stores have been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int done = __hip_atomic_fetch_add(&a.tickets[(long long)r * a.nkv + kvh], 1, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+    last_block = done == s_last - s_first;
+  }
+  __syncthreads();
+  if (!last_block) return;
+  for (int idx = threadIdx.x; idx < HD * G; idx += NW * 64) {
+    const int d = idx / G, c = idx - d * G;
+    const int hh = kvh * G + c;
+    const long long base = ((long long)r * a.nh + hh) * a.nsplit;
+    // four splits' values are asked for together; the sum runs in ascending split order under a
+    // running maximum
+    float M = -INFINITY, acc = 0.f, L = 0.f;
+    for (int s0 = s_first; s0 <= s_last; s0 += 4) {
+      float pm[4], pl[4], po[4];
 #pragma unroll
-  for (int j = 0; j < HD / 64 + 1; ++j) acc[j] = 0.f;
-  for (int s = s_first; s <= s_last; ++s) {
-    const float wgt = exp2f(a.part_ml[(base + s) * 2] - M);
-    L += wgt * a.part_ml[(base + s) * 2 + 1];
+      for (int j = 0; j < 4; ++j) {
+        const long long sp = base + min(s0 + j, s_last);
+        pm[j] = other_blocks_result(a.part_ml + sp * 2);
+        pl[j] = other_blocks_result(a.part_ml + sp * 2 + 1);
+        po[j] = other_blocks_result(a.part_o + sp * HD + d);
+      }
 #pragma unroll
-    for (int j = 0; j < HD / 64 + 1; ++j) {
-      const int d = lane + 64 * j;
-      if (d < HD) acc[j] += wgt * a.part_o[(base + s) * HD + d];
+      for (int j = 0; j < 4; ++j) {
+        if (s0 + j > s_last || pm[j] == -INFINITY) continue;  // (a split whose keys the window hides)
+        const float m_new = fmaxf(M, pm[j]);
+        const float keep = exp2f(M - m_new), wgt = exp2f(pm[j] - m_new);
+        acc = acc * keep + wgt * po[j];
+        L = L * keep + wgt * pl[j];
+        M = m_new;
+      }
     }
+    a.out[(long long)r * a.ldo + hh * HD + d] = f32_to_bf16(acc / L);
   }
-  const float inv = 1.0f / L;
-#pragma unroll
-  for (int j = 0; j < HD / 64 + 1; ++j) {
-    const int d = lane + 64 * j;
-    if (d < HD) a.out[(long long)r * a.ldo + h * HD + d] = f32_to_bf16(acc[j] * inv);
-  }
+  if (threadIdx.x == 0)  // for the next launch
+    __hip_atomic_store(&a.tickets[(long long)r * a.nkv + kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int HD>
@@ -648,37 +724,15 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
     if (G >= 2) return launch_rows<HD, QT, 2>(a, rows, lq_ceil_div(G, 2), stream);
     return launch_rows<HD, QT, 1>(a, rows, 1, stream);
   }
-  // as many waves (at most 16) as keep the partial outputs within 48 KiB of LDS
+  // Four waves a block (two where their partial outputs would not fit 48 KiB of LDS): small blocks
+  // of which a compute unit holds several, each wave with one chunk in flight.
   const int per_wave = (HD * G + 2 * G) * (int)sizeof(float);
-  const int fit = (48 * 1024) / per_wave;
   dim3 grid(a.batch, a.nkv, a.nsplit);
-  // (head sizes above 128 keep to 4 waves: a block of 256 threads may use the whole register file, and
-  // these sizes need more than half of it for one chunk in flight and one being multiplied)
-  bool launched = false;
-  if constexpr (HD <= 64) {
-    if (fit >= 16) {
-      attn_heads_kernel<HD, 16><<<grid, 16 * 64, (size_t)16 * per_wave, stream>>>(a);
-      launched = true;
-    }
-  }
-  if constexpr (HD <= 128) {
-    if (!launched && fit >= 8) {
-      attn_heads_kernel<HD, 8><<<grid, 8 * 64, (size_t)8 * per_wave, stream>>>(a);
-      launched = true;
-    }
-  }
-  if (!launched) {
-    if (fit >= 4)
-      attn_heads_kernel<HD, 4><<<grid, 4 * 64, (size_t)4 * per_wave, stream>>>(a);
-    else
-      attn_heads_kernel<HD, 2><<<grid, 2 * 64, (size_t)2 * per_wave, stream>>>(a);
-  }
+  if (4 * per_wave <= 48 * 1024)
+    attn_heads_kernel<HD, 4><<<grid, 4 * 64, (size_t)4 * per_wave, stream>>>(a);
+  else
+    attn_heads_kernel<HD, 2><<<grid, 2 * 64, (size_t)2 * per_wave, stream>>>(a);
   LQ_CHECK_LAUNCH("attention(mfma heads)");
-  if (a.nsplit > 1) {
-    dim3 mgrid(a.batch, a.nh);
-    attn_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(a);
-    LQ_CHECK_LAUNCH("attention(mfma merge)");
-  }
   return 0;
 }
 
@@ -694,9 +748,17 @@ bool lq_attention_mfma_accepts(int dtype, int nh, int nkv, int hd, int block_siz
   return true;
 }
 
+// Positions per block of a decoding launch.  It depends on the bound rounded up to 1024, so that
+// launches whose bounds differ less than that add up their sums in the same order.
+static int decode_split_len(int rows, int nkv, int max_len) {
+  const long long bound = (long long)lq_ceil_div(max_len, 1024) * 1024;
+  const long long per = ((long long)rows * nkv * bound + 256LL * MAX_DECODE_BLOCKS - 1) / (256LL * MAX_DECODE_BLOCKS);
+  return (int)(256 * (per > 1 ? per : 1));
+}
+
 // Floats of workspace a decode launch needs (0 when one split is enough).
-long long lq_attention_mfma_workspace(int rows, int nh, int hd, int max_len) {
-  const int nsplit = lq_ceil_div(max_len, SPLIT);
+long long lq_attention_mfma_workspace(int rows, int nh, int nkv, int hd, int max_len) {
+  const int nsplit = lq_ceil_div(max_len, decode_split_len(rows, nkv, max_len));
   if (nsplit <= 1) return 0;
   return (long long)rows * nh * nsplit * (hd + 2);
 }
@@ -705,8 +767,8 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
                       int hd, const int* row_pos, const int* seq_slot, const int* cu_rows,
                       const int* block_table, int bt_stride, const void* kcache, const void* vcache,
                       float scale, int window, int decode, int max_len, float* workspace,
-                      long long workspace_floats, const void* k_new, const void* v_new, int ldk, int ldv,
-                      const float* cs, hipStream_t stream) {
+                      long long workspace_floats, int* tickets, long long tickets_n, const void* k_new,
+                      const void* v_new, int ldk, int ldv, const float* cs, hipStream_t stream) {
   AttnArgs a;
   a.q = (const bf16_t*)q;
   a.ldq = ldq;
@@ -727,6 +789,8 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
   a.part_o = nullptr;
   a.part_ml = nullptr;
   a.nsplit = 1;
+  a.split_len = 256;
+  a.tickets = tickets;
   a.k_new = (const bf16_t*)k_new;
   a.v_new = (const bf16_t*)v_new;
   a.ldk = ldk;
@@ -740,12 +804,16 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
   if (decode) {
     LQ_REQUIRE(rows == batch, "attention: decoding needs one row a sequence (%d rows, %d sequences)", rows, batch);
     LQ_REQUIRE(max_len > 0, "attention: decoding needs the longest sequence length");
-    a.nsplit = lq_ceil_div(max_len, SPLIT);
+    a.split_len = decode_split_len(rows, nkv, max_len);
+    a.nsplit = lq_ceil_div(max_len, a.split_len);
     LQ_REQUIRE(a.nsplit <= 65535, "attention: %d tokens are too many splits", max_len);
     if (a.nsplit > 1) {
-      const long long need = lq_attention_mfma_workspace(rows, nh, hd, max_len);
+      const long long need = lq_attention_mfma_workspace(rows, nh, nkv, hd, max_len);
       LQ_REQUIRE(workspace != nullptr && workspace_floats >= need,
                  "attention: workspace of %lld floats needed, %lld given", need, workspace_floats);
+      LQ_REQUIRE(tickets != nullptr && tickets_n >= (long long)rows * nkv,
+                 "attention: %lld ticket counters needed for %d rows and %d kv heads, %lld given",
+                 (long long)rows * nkv, rows, nkv, tickets_n);
       a.part_o = workspace;
       a.part_ml = workspace + (long long)rows * nh * a.nsplit * hd;
     }

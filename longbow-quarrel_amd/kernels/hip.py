@@ -70,6 +70,9 @@ class HipKernels:
             raise KernelLibraryError("no HIP device is visible; this library runs on a gfx950 GPU only")
         self._stream: Optional[int] = None
         self.force_generic = False  # route linear and attention to the size-agnostic kernels
+        # ticket counters of the decoding attention (one for each row and kv head of a launch); a launch
+        # finds them zero and leaves them zero, so launches through one object must not overlap
+        self._tickets = torch.zeros(1 << 18, dtype=torch.int32, device="cuda")
 
     # ------------------------------------------------------------------ plumbing
     def use_stream(self, stream: Optional["torch.cuda.Stream"]) -> None:
@@ -431,7 +434,7 @@ class HipKernels:
             _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(cu_rows), _ptr(block_table),
             c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
             c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
-            c_longlong(ws_n), _ptr(k_new if cos_sin is not None else None),
+            c_longlong(ws_n), _ptr(self._tickets), c_longlong(self._tickets.numel()), _ptr(k_new if cos_sin is not None else None),
             _ptr(v_new if cos_sin is not None else None), c_int(ldk), c_int(ldv), _ptr(cos_sin),
             c_int(1 if self.force_generic else 0), self.stream))
 

@@ -326,6 +326,22 @@ def test_attention_window_edge(kn, dtype, generic, window):
     assert rel_err(got, want) < (2e-6 if dtype == torch.float32 else 8e-3)
 
 
+@pytest.mark.parametrize("head_dim,heads,kv_heads", [(128, 8, 2), (64, 3, 3), (192, 2, 1)])
+@pytest.mark.parametrize("window", [0, 257, 600])
+def test_decode_attention_over_several_splits(kn, head_dim, heads, kv_heads, window):
+    """Rows whose keys lie in up to six splits of 256 positions, the first of them hidden by the window for
+    some rows; a row's splits are added up by whichever of its workgroups comes last, and the counters that
+    tell which one that is are left at zero for the next launch (so the same launch again gives the same)."""
+    lengths = [1500, 900, 256, 257, 64, 1100]
+    got, want = run_attention(kn, None, lengths, [1] * len(lengths), heads, kv_heads, head_dim, torch.bfloat16, 31,
+                              window=window, decode=True)
+    assert rel_err(got, want) < 8e-3
+    again, _ = run_attention(kn, None, lengths, [1] * len(lengths), heads, kv_heads, head_dim, torch.bfloat16, 31,
+                             window=window, decode=True)
+    assert torch.equal(got, again)
+    assert int(kn._tickets.abs().max()) == 0
+
+
 @pytest.mark.parametrize("dtype,generic", [(torch.float32, True), (torch.bfloat16, False)])
 @pytest.mark.parametrize("decode", [False, True])
 def test_attention_finds_one_far_key_among_hundreds(kn, dtype, generic, decode):
