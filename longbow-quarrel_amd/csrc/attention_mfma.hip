@@ -319,17 +319,26 @@ struct RowsLds {
   static constexpr int PIECES = HD * 8;          // 16-byte pieces of K (and of V^T) in one cache block
 };
 
-template <int HD, int QT, int NW>
-__global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_rows_kernel(AttnArgs a, int heads_per_block_group) {
+template <int HD, int QT, int HW, int RT>
+__global__ __launch_bounds__(HW * RT * 64, (HD <= 128 && HW * RT > 1 ? 2 : 1)) void attn_rows_kernel(AttnArgs a, int heads_per_block_group, int tiles, int units) {
   using L = RowsLds<HD>;
-  constexpr int ROWS = QT * 16;
+  constexpr int NW = HW * RT;  // wave = row group * HW + head: HW query heads of one kv head, RT groups of QT row tiles
+  constexpr int ROWS = QT * 16 * RT;
   constexpr int THREADS = NW * 64;
   constexpr int PER_THREAD = (L::PIECES + THREADS - 1) / THREADS;  // pieces of K, and of V, per thread
+  constexpr bool EARLY = PER_THREAD <= 8;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-  // find this block's tile: tiles of ROWS rows, counted sequence by sequence.  Blocks are taken from
-  // the back: a sequence's late tiles see the most keys and should start first.
-  int t = gridDim.x - 1 - blockIdx.x, b = 0, r0 = -1, nrows = 0;
+  // Tasks (a tile of ROWS rows, counted sequence by sequence, for one group of heads) in descending
+  // order of their keys: late tiles first.  Workgroups i, i + units, i + 2 units, ... land on the
+  // same compute unit, so the tasks are dealt out in a snake (0 .. units-1, then back): a unit's
+  // heavy task gets a light partner and the units finish together.
+  const int per_tile = gridDim.x / tiles;  // groups of heads
+  const int round = blockIdx.x / units, place = blockIdx.x % units;
+  int task = round * units + ((round & 1) ? units - 1 - place : place);
+  if ((round + 1) * units > (int)gridDim.x) task = blockIdx.x;  // the last, partial round stays in order
+  const int head_group = task % per_tile;
+  int t = tiles - 1 - task / per_tile, b = 0, r0 = -1, nrows = 0;
   for (; b < a.batch; ++b) {
     const int begin = a.cu_rows[b], n = a.cu_rows[b + 1] - begin;
     const int tiles = (n + ROWS - 1) / ROWS;
@@ -343,9 +352,10 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_r
   if (r0 < 0) return;  // the whole block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c16 = lane & 15, g = lane >> 4;
   const int G = a.nh / a.nkv;
-  // blockIdx.y = kv head * groups + group, a group being NW consecutive query heads of the kv head
-  const int kvh = blockIdx.y / heads_per_block_group;
-  const int hq = (blockIdx.y % heads_per_block_group) * NW + wave;
+  // blockIdx.y = kv head * groups + group, a group being HW consecutive query heads of the kv head
+  const int kvh = head_group / heads_per_block_group;
+  const int hq = (head_group % heads_per_block_group) * HW + wave % HW;
+  const int tile0 = (wave / HW) * QT;  // this wave's first row tile within the block
   const bool wave_active = hq < G;  // an idle wave still copies and meets the barriers
   const int h = kvh * G + min(hq, G - 1);
   const int* table = a.block_table + (long long)a.seq_slot[b] * a.bt_stride;
@@ -355,18 +365,18 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_r
   init_tiles<HD, QT>(w);
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
-    const int rows_here = min(16, nrows - qt * 16);  // may be <= 0: the tile is empty
-    const int rc = qt * 16 + min(c16, max(rows_here, 1) - 1);
+    const int rows_here = min(16, nrows - (tile0 + qt) * 16);  // may be <= 0: the tile is empty
+    const int rc = (tile0 + qt) * 16 + min(c16, max(rows_here, 1) - 1);
     const int row = r0 + min(rc, nrows - 1);
     w.valid[qt] = wave_active && c16 < rows_here;
     w.pos[qt] = p0 + min(rc, nrows - 1);
     w.lo[qt] = (a.window > 0 && w.pos[qt] >= a.window) ? w.pos[qt] - a.window + 1 : 0;
-    const int first_pos = p0 + min(qt * 16, nrows - 1);
-    w.last_key[qt] = (wave_active && rows_here > 0) ? p0 + qt * 16 + rows_here - 1 : -1;
+    const int first_pos = p0 + min((tile0 + qt) * 16, nrows - 1);
+    w.last_key[qt] = (wave_active && rows_here > 0) ? p0 + (tile0 + qt) * 16 + rows_here - 1 : -1;
     w.first_key[qt] = (a.window > 0 && first_pos >= a.window) ? first_pos - a.window + 1 : 0;
     // a full tile of 16 rows: keys up to its first row's position and from its last row's window
     // start on are visible to all of its columns
-    const int last_pos = p0 + qt * 16 + rows_here - 1;
+    const int last_pos = p0 + (tile0 + qt) * 16 + rows_here - 1;
     w.free_to[qt] = (wave_active && rows_here == 16) ? first_pos : -1;
     w.free_from[qt] = (a.window > 0 && last_pos >= a.window) ? last_pos - a.window + 1 : 0;
     const bf16_t* qr = a.q + (long long)row * a.ldq + h * HD + g * 8;
@@ -426,6 +436,9 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_r
     unsigned char* cur = smem + ((lb - blk_first) & 1) * L::STAGE;
     unsigned char* nxt = smem + ((lb - blk_first + 1) & 1) * L::STAGE;
     const bool more = lb < blk_last;
+    // The next block's loads are on their way during this block's products where a thread's share
+    // of them is small enough to stay in registers meanwhile; else they follow the products.
+    if (EARLY && more) fetch(lb + 1);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int t0 = lb * BS + half * 32;
@@ -461,12 +474,9 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_r
         }
       }
     }
-    // The next block is copied after this one's products: its registers are then not live across them,
-    // which keeps a wave within half the register file, and the copy's latency is covered by the
-    // other block resident on the compute unit.  Nobody reads nxt: its last readers passed the
-    // barrier below one round ago.
+    // Nobody reads nxt: its last readers passed the barrier below one round ago.
     if (more) {
-      fetch(lb + 1);
+      if (!EARLY) fetch(lb + 1);
       stash(lb + 1, nxt);
     }
     __syncthreads();
@@ -477,7 +487,7 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_r
     l = rows_sum(l);
     if (!w.valid[qt]) continue;
     const float inv = 1.0f / l;
-    bf16_t* orow = a.out + (long long)(r0 + qt * 16 + c16) * a.ldo + h * HD + g * 4;
+    bf16_t* orow = a.out + (long long)(r0 + (tile0 + qt) * 16 + c16) * a.ldo + h * HD + g * 4;
 #pragma unroll
     for (int dt = 0; dt < HD / 16; ++dt) {
       u32x2 ww;
@@ -488,12 +498,12 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 && NW > 1 ? 2 : 1)) void attn_r
   }
 }
 
-template <int HD, int QT, int NW>
+template <int HD, int QT, int HW, int RT>
 int launch_rows(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
   using L = RowsLds<HD>;
-  constexpr int ROWS = QT * 16;
+  constexpr int ROWS = QT * 16 * RT, NW = HW * RT;
   const size_t smem = 2 * (size_t)L::STAGE;
-  auto kernel = attn_rows_kernel<HD, QT, NW>;
+  auto kernel = attn_rows_kernel<HD, QT, HW, RT>;
   static bool configured = false;
   if (!configured && smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -503,8 +513,8 @@ int launch_rows(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
     }
     configured = true;
   }
-  dim3 grid(lq_ceil_div(rows, ROWS) + a.batch, a.nkv * groups);
-  kernel<<<grid, NW * 64, smem, stream>>>(a, groups);
+  const int tiles = lq_ceil_div(rows, ROWS) + a.batch;  // an upper bound: a sequence's last tile may be partial
+  kernel<<<dim3(tiles * a.nkv * groups), NW * 64, smem, stream>>>(a, groups, tiles, lq_compute_units());
   LQ_CHECK_LAUNCH("attention(mfma rows)");
   return 0;
 }
@@ -720,9 +730,10 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
   const int G = a.nh / a.nkv;
   if (!decode) {
     constexpr int QT = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
-    if (G >= 4) return launch_rows<HD, QT, 4>(a, rows, lq_ceil_div(G, 4), stream);
-    if (G >= 2) return launch_rows<HD, QT, 2>(a, rows, lq_ceil_div(G, 2), stream);
-    return launch_rows<HD, QT, 1>(a, rows, 1, stream);
+    constexpr int QT2 = QT > 1 ? QT / 2 : 1;  // with two row groups of waves: the same rows a block, half a wave
+    if (G >= 4) return launch_rows<HD, QT2, 4, 2>(a, rows, lq_ceil_div(G, 4), stream);
+    if (G >= 2) return launch_rows<HD, QT, 2, 1>(a, rows, lq_ceil_div(G, 2), stream);
+    return launch_rows<HD, QT, 1, 1>(a, rows, 1, stream);
   }
   // Four waves a block (two where their partial outputs would not fit 48 KiB of LDS): small blocks
   // of which a compute unit holds several, each wave with one chunk in flight.

@@ -105,6 +105,7 @@ __device__ inline float block_max(float v, float* smem) {
 // ---- error reporting ---------------------------------------------------------
 
 void lq_set_error(const char* fmt, ...);
+int lq_compute_units();  // of the current device
 
 #define LQ_REQUIRE(cond, ...)   \
   do {                          \

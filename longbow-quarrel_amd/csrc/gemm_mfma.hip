@@ -676,18 +676,6 @@ __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16
   }
 }
 
-static int lq_compute_units() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      n = prop.multiProcessorCount;
-    if (n <= 0) n = 256;
-  }
-  return n;
-}
-
 // How many blocks should share K for an [M, K] x [N, K]^T product with the balanced kernel (1: no
 // split).  With several row tiles a block wants several column tiles too, so that the x fragments it
 // holds are used more than once; a matrix with few columns gets them by giving each block a wider run
@@ -792,8 +780,8 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
     // a wider one leaves part empty.  Cost of a round relative to the 256-column tile, as measured.
     const int cus = lq_compute_units(), tm = lq_ceil_div(M, 256);
     const double c256 = 1.00 * lq_ceil_div(tm * lq_ceil_div(N, 256), cus);
-    const double c224 = 0.96 * lq_ceil_div(tm * lq_ceil_div(N, 224), cus);
-    const double c192 = 0.79 * lq_ceil_div(tm * lq_ceil_div(N, 192), cus);
+    const double c224 = 1.02 * lq_ceil_div(tm * lq_ceil_div(N, 224), cus);
+    const double c192 = 0.83 * lq_ceil_div(tm * lq_ceil_div(N, 192), cus);
     if (c256 <= c224 && c256 <= c192)
       return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     if (c224 <= c192)

@@ -17,6 +17,19 @@ extern "C" const char* lq_last_error() { return g_error; }
 
 extern "C" int lq_abi_version() { return 1; }
 
+// Compute units of the current device (256 if the runtime will not say).
+int lq_compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      n = prop.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+
 // ---- HIP graphs: capture what a step launches on `stream`, replay it later ----
 // Captured steps must not allocate and must not record memsets; the library's
 // kernels obey both (buffers are cleared by fill kernels).
