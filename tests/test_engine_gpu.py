@@ -272,6 +272,35 @@ def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory
     assert g1.tokens == g2.tokens
 
 
+def test_decoding_batches_that_shrink_from_40_rows_to_one(tmp_path_factory):
+    """40 sequences that end one after the other: decoding steps of 40 down to 1 row take the matrix-vector
+    kernels with four, two and one row tile (K shared between blocks, the pieces added by the norms; below
+    17 rows the norms folded into the products), against the plain implementation."""
+    folder = write_folder(tmp_path_factory.mktemp("wide64"), WIDE, seed=4, std=0.03)
+    eng = lq.load_engine(folder, dtype="bfloat16", max_tokens=64 * 48)
+    c, tensors = read_folder(folder)
+    ref = plain.PlainLlama(c, tensors)
+    reqs = [random_tokens(4 + (i * 7) % 23, WIDE["vocab_size"], 500 + i) for i in range(40)]
+    want = [ref.forward(r, plain.round_bf16) for r in reqs]
+    slots = [eng.new_sequence() for _ in reqs]
+    out = [[] for _ in reqs]
+    first = eng.step([StepEntry(s, r[:3], range(3)) for s, r in zip(slots, reqs)])
+    for i in range(len(reqs)):
+        out[i].append(first[3 * i : 3 * i + 3])
+    pos = 3
+    rows_seen = set()
+    while any(pos < len(r) for r in reqs):
+        live = [i for i, r in enumerate(reqs) if pos < len(r)]
+        rows_seen.add(len(live))
+        got = eng.step([StepEntry(slots[i], [reqs[i][pos]], [0]) for i in live])
+        for j, i in enumerate(live):
+            out[i].append(got[j : j + 1])
+        pos += 1
+    for i, w in enumerate(want):
+        assert rel_err(torch.cat(out[i]), w) < TOL_BF16, i
+    assert any(r > 32 for r in rows_seen) and any(16 < r <= 32 for r in rows_seen) and any(r <= 16 for r in rows_seen)
+
+
 LONG = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermediate_size": 264,
     "num_hidden_layers": 2, "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 128,
