@@ -1,5 +1,6 @@
 """The reference's programmatic interface, in Python's spelling: `NewEngine(path, cfg)`, `Infer`,
-`InferWithCallback`, `InferWithLogits`, `Close` (internal/engine/engine.go:380, 1273-1296) and
+`InferWithCallback`, `InferWithLogits`, `Close`, `GetEmbedding(s)`, `EmbeddingDim`
+(internal/engine/engine.go:380, 1273-1296, 1809-1858) and
 `SamplerConfig{Temperature, TopK, TopP, RepPenalty, Seed}` (internal/engine/types_base.go:7-15).
 One sequence a call, as there; batches go through `generate`."""
 from __future__ import annotations
@@ -67,6 +68,28 @@ class QuarrelEngine:
         gave them (before the repetition penalty) (engine.go:1278-1285)."""
         ids, logits = self._run(tokens, n, sampler_config, None, True)
         return ids, logits[0]
+
+    def embedding_dim(self) -> int:
+        """Width of the embedding vectors (engine.go:1852-1858)."""
+        return int(self.engine.model.spec.width)
+
+    def get_embeddings(self, tokens: Sequence[int]) -> torch.Tensor:
+        """The rows of the embedding table for these ids, float32 [len(tokens), width], looked up by
+        the kernel the model itself starts with (engine.go:1809-1836)."""
+        e = self.engine
+        vocab = int(e.model.spec.vocab_size)
+        for i, t in enumerate(tokens):
+            if not 0 <= int(t) < vocab:
+                raise ValueError(f"token {t} (place {i}) out of vocab range [0, {vocab})")  # engine.go:1814-1816
+        ids = torch.tensor([int(t) for t in tokens], dtype=torch.int32, device=e.device)
+        out = torch.empty((len(tokens), self.embedding_dim()), dtype=torch.float32, device=e.device)
+        if len(tokens):
+            e.run_on_stream(lambda: e.kernels.embed(e.model.embedding, ids, out))
+        return out
+
+    def get_embedding(self, token: int) -> torch.Tensor:
+        """One id's embedding vector, float32 [width] (engine.go:1809-1822)."""
+        return self.get_embeddings([token])[0]
 
     def close(self) -> None:
         self.engine = None

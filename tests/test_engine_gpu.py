@@ -347,7 +347,7 @@ def test_a_sequence_longer_than_one_split_of_decode_attention(tmp_path_factory, 
 
 def test_the_reference_style_interface(tmp_path_factory):
     """new_engine / infer / infer_with_callback / infer_with_logits / close (internal/engine/engine.go:380,
-    1273-1296) give what `generate` gives for one sequence."""
+    1273-1296) give what `generate` gives for one sequence; the embedding look-ups give the table's rows."""
     eng, ref, act, reqs, want, folder = setup_case(tmp_path_factory, "b", "float32")
     prompt = reqs[2][:12]
     q = lq.new_engine(folder, dtype="float32", kv_cache_size=256)
@@ -361,6 +361,14 @@ def test_the_reference_style_interface(tmp_path_factory):
     assert rel_err(logits, whole[-1]) < TOL_F32  # the logits the last id was taken from
     cfg = lq.SamplerConfig(temperature=0.8, top_k=40, top_p=0.95, rep_penalty=1.1, seed=4)
     assert q.infer(prompt, 9, cfg) == lq.generate(eng, [prompt], 9, cfg.params(), stop_ids=[5, 7]).tokens[0]
+    # GetEmbedding(s) / EmbeddingDim (engine.go:1809-1858): rows of the table as they are stored
+    _, tensors = read_folder(folder)
+    table = tensors["model.embed_tokens.weight"].float()
+    assert q.embedding_dim() == TINY_B["hidden_size"] == table.shape[1]
+    assert torch.equal(q.get_embeddings([5, 0, 383]).cpu(), table[[5, 0, 383]])
+    assert torch.equal(q.get_embedding(17).cpu(), table[17])
+    with pytest.raises(ValueError, match="out of vocab range"):
+        q.get_embedding(TINY_B["vocab_size"])
     q.close()
 
 
