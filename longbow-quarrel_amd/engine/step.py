@@ -131,13 +131,14 @@ class Engine:
         torch.cuda.current_stream(self.device).wait_stream(self.stream)
         return out
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], observe=None) -> Optional[torch.Tensor]:
         """Runs the entries' tokens; returns float32 logits [wanted, vocab] in the order of the
-        entries and of each entry's `want` (None if nothing is wanted)."""
+        entries and of each entry's `want` (None if nothing is wanted).  `observe(name, x, pending)`, for
+        debugging, sees the residual stream after the embedding and after every run of the schedule."""
         self._validate(entries)
-        return self.run_on_stream(lambda: self._step(entries))
+        return self.run_on_stream(lambda: self._step(entries, observe))
 
-    def _step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _step(self, entries: Sequence[StepEntry], observe=None) -> Optional[torch.Tensor]:
         cache = self.cache
         growth = {e.slot: len(e.tokens) for e in entries}
         cache.reserve(growth)  # CacheFull leaves everything as it was
@@ -169,7 +170,7 @@ class Engine:
             seq_slot=d_slot, seq_start=d_start, seq_len=d_len, cu_rows=d_cu,
             host_slots=slots, host_start=starts, host_new=[len(e.tokens) for e in entries],
             max_new=max(len(e.tokens) for e in entries), max_len=max(lens),
-            decode=all(len(e.tokens) == 1 for e in entries),
+            decode=all(len(e.tokens) == 1 for e in entries), observe=observe,
         )
         logits = self.model.forward(ctx, cache.layer_views(), d_want, len(want_rows))
         cache.advance(growth)

@@ -103,6 +103,8 @@ class DecoderModel:
         x = ctx.ws.alloc((ctx.rows, s.width), torch.float32, keep=True)
         kn.embed(self.embedding, ctx.tokens, x)
         pending: Optional[torch.Tensor] = None
+        if ctx.observe is not None:
+            ctx.observe("embed", x, None)
         for i, run in enumerate(s.schedule):
             ctx.ws.next_run()  # the buffers of the run before the last one are free again
             cache = caches.get(i if run.cache_of is None else run.cache_of)
@@ -115,6 +117,8 @@ class DecoderModel:
                 pending = block.forward(x, pending, ctx, cache, next_norm=after)
             else:
                 pending = block.forward(x, pending, ctx, cache)
+            if ctx.observe is not None:
+                ctx.observe(f"run {i}", x, None if isinstance(pending, RowStats) else pending)
         if n_want == 0:
             return None
         ctx.ws.next_run()

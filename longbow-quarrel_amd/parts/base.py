@@ -226,6 +226,10 @@ class StepContext:
     decode: bool = False  # every sequence brings exactly one token
     logits_out: Optional[torch.Tensor] = None  # where the logits go (a captured step's fixed buffer)
     shared: Dict[Any, Any] = field(default_factory=dict)  # what parts compute once a step and share
+    # debugging: called with ("embed" | "run <i>", x, pending) after the embedding and after every run of the
+    # schedule; the residual stream at that point is x plus what is pending (a delta, pieces of one, or
+    # nothing when the product has added it already)
+    observe: Optional[Any] = None
 
 
 @dataclass

@@ -17,10 +17,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LENGTHS = (40, 70, 33, 129, 3)
 
 
-def replay(folder, dtype, steps, out_dir, max_tokens):
+def replay(folder, dtype, steps, out_dir, max_tokens, extra=()):
     """Feeds the steps one at a time, each only after the previous `done` line, as a driver would."""
     proc = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-                             "--out", out_dir, "--max-tokens", str(max_tokens)],
+                             "--out", out_dir, "--max-tokens", str(max_tokens), *extra],
                             stdin=subprocess.PIPE, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
     try:
         for st in steps:
@@ -117,6 +117,29 @@ def test_replay_whole_tail_and_batched(models, tmp_path, name, dtype):
     for step, w in expect:
         assert rel_err(read_step(out, step, vocab), w) < tol, step
     assert not os.path.exists(os.path.join(out, "1.f32"))  # nothing was wanted in step 1
+
+
+def test_replay_dumps_the_residual_stream_after_every_layer(models, tmp_path):
+    """--dump-activations: the stream after the embedding and after each layer, for a prompt step and for a
+    decoding step (where the products add into the stream themselves), against the plain layers."""
+    folder, cfg, ref, reqs = models["b"]
+    toks = reqs["r0"]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:-1], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[-1:], "want": [0]}], "end": ["a"]}]
+    dump = str(tmp_path / "acts")
+    replay(folder, "float32", steps, str(tmp_path / "o"), 64, extra=["--dump-activations", dump])
+    emb = ref.w("model.embed_tokens.weight")
+    x = emb[torch.tensor(toks, dtype=torch.long)]
+    width = cfg["hidden_size"]
+
+    def dumped(step, name):
+        return torch.from_numpy(np.fromfile(os.path.join(dump, f"{step}.{name}.f32"), dtype="<f4").reshape(-1, width).copy())
+
+    assert rel_err(dumped(0, "embed"), x[:-1]) < 1e-6 and rel_err(dumped(1, "embed"), x[-1:]) < 1e-6
+    for layer in range(cfg["num_hidden_layers"]):
+        x = ref.decoder_layer(layer, x, plain.identity)
+        assert rel_err(dumped(0, f"run{layer}"), x[:-1]) < TOL_F32, layer
+        assert rel_err(dumped(1, f"run{layer}"), x[-1:]) < TOL_F32, layer
 
 
 def test_replay_refuses_more_tokens_than_the_cache_was_sized_for(models, tmp_path):
