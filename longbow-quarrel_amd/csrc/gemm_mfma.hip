@@ -40,6 +40,13 @@ __device__ inline bf16x8 as_bf16x8(u32x4 v) {
   return c.b;
 }
 
+// A pointer that is the same in every lane, held in scalar registers.
+__device__ inline const char* uniform_ptr(const char* p) {
+  const unsigned long long v = (unsigned long long)p;
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+  return (const char*)(((unsigned long long)hi << 32) | lo);
+}
+
 template <typename TO>
 __device__ inline void store_out(TO* p, float v);
 template <>
@@ -276,13 +283,14 @@ struct PipeShape {
   static constexpr int A_BYTES = BM * ROW_BYTES, STAGE_BYTES = (BM + BN) * ROW_BYTES;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static constexpr int KK = BK / 16;                        // 16-k steps a slab
-  static_assert(BM % ROWS_PER_DMA == 0 && BN % ROWS_PER_DMA == 0, "a transfer must not straddle A and W");
+  static_assert(BM % (ROWS_PER_DMA * NW) == 0 && BN % ROWS_PER_DMA == 0, "whole rounds of transfers for A, then W");
+  static constexpr int A_ROUNDS = BM / (ROWS_PER_DMA * NW);  // transfers j < A_ROUNDS of every wave fetch A
   static_assert(DMA * (STAGES - 1) < 64, "vmcnt has 6 bits");
   // chunk position of chunk c in row r: rows that share a 256-byte bank row get different positions
   __device__ static int swizzle(int row) { return (row / (256 / ROW_BYTES)) & (CPR - 1); }
 };
 
-template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO>
+template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO, bool ALTERNATE = false>
 __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw, TO* __restrict__ C, int ldc, int M,
     int N, int K, int tiles_m, int tiles_n, int k_share, long long split_stride) {
@@ -302,22 +310,28 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
   const int wm = wave / GN, wn = wave % GN;
 
   // where this lane's 16 bytes of each transfer come from: transfer x = NW j + wave fills the stage's
-  // chunks [64 x, 64 x + 64); chunk p is stage row p / CPR (A rows first), position p % CPR
-  const bf16_t* src[S::DMA];
+  // chunks [64 x, 64 x + 64); chunk p is stage row p / CPR (A rows first), position p % CPR.  The address
+  // is a wave-uniform origin (the operand's tile at this block's first k) plus a 32-bit lane offset.
+  const char* a_origin = (const char*)(A + (long long)m0 * lda + k_begin);
+  const char* w_origin = (const char*)(W + (long long)n0 * ldw + k_begin);
+  unsigned off[S::DMA];
   int dst[S::DMA];
 #pragma unroll
   for (int j = 0; j < S::DMA; ++j) {
     const int x = min(j * S::NW + wave, S::TRANSFERS - 1);
     const int p = x * 64 + lane, row = p / S::CPR, c = (p % S::CPR) ^ S::swizzle(row);
-    src[j] = (row < S::BM ? A + (long long)min(m0 + row, M - 1) * lda : W + (long long)min(n0 + row - S::BM, N - 1) * ldw) +
-             k_begin + c * 8;
+    off[j] = row < S::BM ? (unsigned)(min(m0 + row, M - 1) - m0) * (unsigned)lda * 2u + c * 16
+                         : (unsigned)(min(n0 + row - S::BM, N - 1) - n0) * (unsigned)ldw * 2u + c * 16;
     dst[j] = x * 1024;
   }
   auto dma = [&](int stage, int k0) {
     unsigned char* base = plds + stage * S::STAGE_BYTES;
 #pragma unroll
-    for (int j = 0; j < S::DMA; ++j)
-      __builtin_amdgcn_global_load_lds(LQ_GLOBAL_PTR(src[j] + k0), LQ_LDS_PTR(base + dst[j]), 16, 0, 0);
+    for (int j = 0; j < S::DMA; ++j) {
+      // a scalar base and a 32-bit lane offset: one address register a transfer
+      const char* origin = uniform_ptr((j < S::A_ROUNDS ? a_origin : w_origin) + (long long)k0 * 2);
+      __builtin_amdgcn_global_load_lds(LQ_GLOBAL_PTR(origin + off[j]), LQ_LDS_PTR(base + dst[j]), 16, 0, 0);
+    }
   };
 
   // fragment addresses within a 32-row group: row lane % 32, chunk 2 kk + lane / 32, swizzled
@@ -337,9 +351,6 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   const int slabs = k_share / BK;
-#pragma unroll
-  for (int q = 0; q < STAGES - 1; ++q)
-    if (q < slabs) dma(q, q * BK);
 
   auto step = [&](int stage, int t) {
     // this wave's transfers of slab t have landed (those of the slabs behind it may still fly) ...
@@ -378,10 +389,73 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     }
   };
   static_assert(STAGES >= 2 && STAGES <= 4, "the wait above knows 2 to 4 stages");
-  for (int t = 0; t < slabs; t += STAGES) {
+  if constexpr (!ALTERNATE) {
 #pragma unroll
-    for (int q = 0; q < STAGES; ++q)
-      if (t + q < slabs) step(q, t + q);
+    for (int q = 0; q < STAGES - 1; ++q)
+      if (q < slabs) dma(q, q * BK);
+    for (int t = 0; t < slabs; t += STAGES) {
+#pragma unroll
+      for (int q = 0; q < STAGES; ++q)
+        if (t + q < slabs) step(q, t + q);
+    }
+  } else {
+    // Two groups of four waves (one wave of each on every SIMD) take turns: while one group multiplies
+    // slab t, the other reads its fragments of slab t (or t + 1) from LDS, so the matrix pipe and the LDS
+    // port of a SIMD work at the same time.  Every wave runs  fetch(t) | barrier | multiply(t) | barrier;
+    // the second group has passed one barrier more before it starts, which puts it half a period behind.
+    // Who may overwrite what: slab t is read by group 0 before its barrier X(t) and by group 1 before its
+    // X'(t), which is group 0's Y(t).  So after Y(t) (group 0: start of fetch(t + 1); group 1: start of
+    // multiply(t)) both ask for slab t + 2 into slab t's stage, and both wait for their own transfers of
+    // it two phases later, before the barrier that precedes the first read of slab t + 2 (group 0: end of
+    // multiply(t + 1); group 1: end of fetch(t + 1)).
+    static_assert(!ALTERNATE || (STAGES == 2 && S::NW == 8), "two stages, two groups of four waves");
+    const int group = wave >> 2;
+    dma(0, 0);
+    if (slabs > 1) {
+      dma(1, BK);
+      LQ_WAIT_VMCNT(S::DMA);
+    } else {
+      LQ_WAIT_VMCNT(0);
+    }
+    asm volatile("s_barrier" ::: "memory");             // slab 0 is there
+    if (group == 1) asm volatile("s_barrier" ::: "memory");  // half a period behind
+    auto turn = [&](int stage, int t) {
+      const unsigned char* as = a_base + stage * S::STAGE_BYTES;
+      const unsigned char* ws = w_base + stage * S::STAGE_BYTES;
+      if (group == 0 && t >= 1 && t + 1 < slabs) dma(stage ^ 1, (t + 1) * BK);
+      bf16x8 a[S::KK][WM], b[S::KK][WN];
+#pragma unroll
+      for (int kk = 0; kk < S::KK; ++kk) {
+#pragma unroll
+        for (int i = 0; i < WM; ++i) a[kk][i] = as_bf16x8(*(const u32x4*)(as + i * 32 * S::ROW_BYTES + frag[kk]));
+#pragma unroll
+        for (int j = 0; j < WN; ++j) b[kk][j] = as_bf16x8(*(const u32x4*)(ws + j * 32 * S::ROW_BYTES + frag[kk]));
+      }
+      if (group == 1) LQ_WAIT_VMCNT(0);
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the fragments are in registers
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_barrier" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      if (group == 1 && t + 2 < slabs) dma(stage, (t + 2) * BK);
+      __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+      for (int kk = 0; kk < S::KK; ++kk)
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_s_setprio(0);
+      if (group == 0) LQ_WAIT_VMCNT(0);
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_barrier" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int t = 0; t < slabs; t += 2) {
+      turn(0, t);
+      if (t + 1 < slabs) turn(1, t + 1);
+    }
+    if (group == 0) asm volatile("s_barrier" ::: "memory");
   }
   if constexpr (sizeof(TO) == 2) {
     constexpr int OUT_BYTES = S::BM * (EPI == EPI_SWIGLU ? S::BN / 2 : S::BN) * 2;
@@ -394,12 +468,12 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
   }
 }
 
-template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO>
+template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO, bool ALTERNATE = false>
 int launch_pipelined(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                      int splits, long long split_stride, hipStream_t stream) {
   using S = PipeShape<GM, GN, WM, WN, BK, STAGES>;
   const int tiles_m = lq_ceil_div(M, S::BM), tiles_n = lq_ceil_div(N, S::BN);
-  auto kernel = gemm_bf16_pipelined_kernel<GM, GN, WM, WN, BK, STAGES, EPI, TO>;
+  auto kernel = gemm_bf16_pipelined_kernel<GM, GN, WM, WN, BK, STAGES, EPI, TO, ALTERNATE>;
   static bool configured = false;
   if (!configured && S::LDS_BYTES > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -415,6 +489,8 @@ int launch_pipelined(const void* A, const void* W, void* C, int M, int N, int K,
   LQ_REQUIRE(splits >= 1 && K % (BK * splits) == 0, "linear: the pipelined kernel needs K to be a multiple of %d",
              BK * splits);
   LQ_REQUIRE(splits == 1 || EPI == EPI_NONE, "linear: no epilogue on partial products");
+  LQ_REQUIRE((long long)lda * 2 * S::BM < (1ll << 31) && (long long)ldw * 2 * S::BN < (1ll << 31),
+             "linear: rows too far apart for the tile's 32-bit offsets");
   kernel<<<dim3((int)blocks, splits), S::NW * 64, S::LDS_BYTES, stream>>>(
       (const bf16_t*)A, lda, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, tiles_m, tiles_n, K / splits, split_stride);
   LQ_CHECK_LAUNCH("linear(mfma pipelined)");
@@ -754,8 +830,8 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
     }
     if (M <= 32) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
     if (M <= 64) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
-    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride,
-                                                        stream);
+    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride,
+                                                              stream);
   }
   // wide enough to give every compute unit a run of columns: the balanced kernel; else the simple one
   const bool wide = N >= 8 * lq_compute_units() && K >= 512;
@@ -783,7 +859,7 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
     const double c224 = 1.02 * lq_ceil_div(tm * lq_ceil_div(N, 224), cus);
     const double c192 = 0.83 * lq_ceil_div(tm * lq_ceil_div(N, 192), cus);
     if (c256 <= c224 && c256 <= c192)
-      return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     if (c224 <= c192)
       return launch_pipelined<8, 1, 1, 7, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     return launch_pipelined<4, 2, 2, 3, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
@@ -808,6 +884,14 @@ extern "C" int lq_debug_gemm_tiled(const void* x, const void* w, void* out, int 
   if (wn == -2) return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
   if (wn == -8) return launch_pipelined<4, 2, 2, 3, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
   if (wn == -9) return launch_pipelined<8, 1, 1, 7, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -12)
+    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -13)
+    return launch_pipelined<4, 2, 2, 3, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -14)
+    return launch_pipelined<4, 2, 1, 4, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
+  if (wn == -15)
+    return launch_pipelined<2, 4, 2, 2, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
   lq_set_error("no such tile");
   return -1;
 }
