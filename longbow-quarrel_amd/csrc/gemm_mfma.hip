@@ -818,7 +818,45 @@ int tiled_splits(int M, int N, int K) {
   return splits;
 }
 
-int mfma_splits(int M, int N, int K) { return M <= 64 ? v3_splits(M, N, K) : tiled_splits(M, N, K); }
+// ---- 33 to 256 rows of a wide matrix: the weights are what is read, once, at the speed of the memory.
+// The pipelined kernel streams them best (transfers of three or four slabs in flight, no registers in
+// between) when its tile covers all rows, so that a weight is read once, and is narrow enough, with K shared
+// out over blocks, for about one block a compute unit: 64 x 128 (8 waves), 128 x 128 (8 waves) or 256 x 128
+// tiles (8 waves) of 4, 4 and 3 stages.  A product that must come out whole (16-bit out, or an epilogue)
+// and has few columns takes the 64-column sibling instead.
+inline bool mid_rows(int M, int N, int K) {
+  return M > 32 && M <= 256 && K % 64 == 0 && K >= 512 && N >= 8 * lq_compute_units();
+}
+
+int mid_splits(int M, int N, int K) {
+  const int tiles = lq_ceil_div(N, 128), want = 3 * lq_compute_units() / 4;
+  int splits = 1;
+  while (splits < 16 && tiles * splits < want && K % (128 * splits) == 0 && K / (2 * splits) >= 512) splits *= 2;
+  return splits;
+}
+
+template <int EPI, typename TO>
+int launch_mid(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc, int splits,
+               long long split_stride, hipStream_t stream) {
+  // whole and with few columns: 64-column tiles (no epilogue pairs columns across them)
+  if constexpr (EPI == EPI_NONE) {
+    if (splits == 1 && lq_ceil_div(N, 128) * 8 < 3 * lq_compute_units()) {
+      if (M <= 64) return launch_pipelined<2, 2, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      if (M <= 128) return launch_pipelined<2, 2, 2, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      return launch_pipelined<4, 2, 2, 1, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    }
+  }
+  if (M <= 64)
+    return launch_pipelined<2, 4, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+  if (M <= 128)
+    return launch_pipelined<4, 2, 1, 2, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+  return launch_pipelined<4, 2, 2, 2, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+}
+
+int mfma_splits(int M, int N, int K) {
+  if (mid_rows(M, N, K)) return mid_splits(M, N, K);
+  return M <= 64 ? v3_splits(M, N, K) : tiled_splits(M, N, K);
+}
 
 template <int EPI, typename TO>
 int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
@@ -828,6 +866,9 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
       lq_set_error("linear: %d shares of K are not what this product takes (%d)", splits, mfma_splits(M, N, K));
       return -1;
     }
+  }
+  if (mid_rows(M, N, K)) return launch_mid<EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+  if (splits > 1) {
     if (M <= 32) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
     if (M <= 64) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
     return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride,
@@ -888,10 +929,6 @@ extern "C" int lq_debug_gemm_tiled(const void* x, const void* w, void* out, int 
     return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
   if (wn == -13)
     return launch_pipelined<4, 2, 2, 3, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
-  if (wn == -14)
-    return launch_pipelined<4, 2, 1, 4, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
-  if (wn == -15)
-    return launch_pipelined<2, 4, 2, 2, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
   lq_set_error("no such tile");
   return -1;
 }

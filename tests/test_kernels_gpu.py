@@ -112,6 +112,9 @@ def test_linear_float32(kn, m, n, k):
     (17, 256, 128), (32, 4096, 4096), (33, 515, 1000), (64, 130, 264), (64, 4096, 14336),  # skinny, more row tiles
     (65, 256, 128), (100, 300, 1000), (128, 128, 64), (257, 515, 4096),                   # tiled
     (2048, 1024, 512),
+    (40, 2048, 512), (48, 2064, 1024), (64, 6144, 4096), (33, 28672, 512),                 # pipelined, 64-row tiles
+    (65, 2048, 512), (128, 4104, 1088), (100, 28672, 512),                                 # pipelined, 128-row tiles
+    (129, 3000, 2048), (256, 2048, 4096), (200, 28672, 512),                               # pipelined, 256 x 128 / 64
     (1000, 12700, 192), (300, 49000, 64), (2048, 6144, 4096),     # pipelined, 256 x 256 tiles
     (1000, 8200, 96), (130, 66000, 32), (2048, 4096, 4000),        # pipelined, 128 x 256 tiles
 ])
@@ -125,7 +128,8 @@ def test_linear_bfloat16_matrix_cores(kn, out_dtype, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 4096, 4096), (17, 4096, 14336), (40, 2560, 2056), (33, 6144, 4096),
-                                   (300, 4096, 4096), (2048, 4096, 14336), (65, 1000, 2048)])
+                                   (300, 4096, 4096), (2048, 4096, 14336), (65, 1000, 2048), (130, 4096, 14336),
+                                   (256, 2100, 1024)])
 def test_linear_in_pieces_and_their_consumers(kn, m, n, k):
     """Few columns and several row tiles: K is shared out over blocks and the product comes as
     pieces; the norm, the add and the row gather that take such a delta add the pieces up."""
@@ -410,7 +414,7 @@ def test_rope_store_rotates_and_writes_the_right_rows(kn, dtype):
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 33, 64, 65, 300, 400])
-@pytest.mark.parametrize("inner,k", [(16, 8), (328, 96), (1000, 264), (8200, 96), (14336, 4096)])
+@pytest.mark.parametrize("inner,k", [(16, 8), (328, 96), (1000, 264), (8200, 96), (14336, 4096), (1032, 512)])
 def test_linear_with_fused_swiglu(kn, m, inner, k):
     """One kernel for silu(x Wg^T) * (x Wu^T), with gate and up rows interleaved in groups of 8
     (every kernel of the product has this epilogue: the GEMVs, the tiled and the pipelined ones)."""
