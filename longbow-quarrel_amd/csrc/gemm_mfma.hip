@@ -822,8 +822,8 @@ int tiled_splits(int M, int N, int K) {
 // The pipelined kernel streams them best (transfers of three or four slabs in flight, no registers in
 // between) when its tile covers all rows, so that a weight is read once, and is narrow enough, with K shared
 // out over blocks, for about one block a compute unit: 64 x 128 (8 waves), 128 x 128 (8 waves) or 256 x 128
-// tiles (8 waves) of 4, 4 and 3 stages.  A product that must come out whole (16-bit out, or an epilogue)
-// and has few columns takes the 64-column sibling instead.
+// tiles (8 waves) of 4, 4 and 3 stages.  A product that must come out whole (16-bit out: its consumer adds no
+// pieces) and has few columns takes the 64- or 32-column sibling instead.
 inline bool mid_rows(int M, int N, int K) {
   return M > 32 && M <= 256 && K % 64 == 0 && K >= 512 && N >= 8 * lq_compute_units();
 }
@@ -838,9 +838,15 @@ int mid_splits(int M, int N, int K) {
 template <int EPI, typename TO>
 int launch_mid(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc, int splits,
                long long split_stride, hipStream_t stream) {
-  // whole and with few columns: 64-column tiles (no epilogue pairs columns across them)
+  // whole and with few columns: 64- or 32-column tiles (no epilogue pairs columns across them)
   if constexpr (EPI == EPI_NONE) {
-    if (splits == 1 && lq_ceil_div(N, 128) * 8 < 3 * lq_compute_units()) {
+    const int want = 3 * lq_compute_units() / 4;
+    if (splits == 1 && lq_ceil_div(N, 64) < want) {
+      if (M <= 64) return launch_pipelined<2, 1, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      if (M <= 128) return launch_pipelined<4, 1, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      return launch_pipelined<8, 1, 1, 1, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    }
+    if (splits == 1 && lq_ceil_div(N, 128) < want) {
       if (M <= 64) return launch_pipelined<2, 2, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
       if (M <= 128) return launch_pipelined<2, 2, 2, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
       return launch_pipelined<4, 2, 2, 1, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);

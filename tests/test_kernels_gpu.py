@@ -115,6 +115,7 @@ def test_linear_float32(kn, m, n, k):
     (40, 2048, 512), (48, 2064, 1024), (64, 6144, 4096), (33, 28672, 512),                 # pipelined, 64-row tiles
     (65, 2048, 512), (128, 4104, 1088), (100, 28672, 512),                                 # pipelined, 128-row tiles
     (129, 3000, 2048), (256, 2048, 4096), (200, 28672, 512),                               # pipelined, 256 x 128 / 64
+    (50, 12800, 512), (100, 12800, 512), (200, 12800, 512),                                # their 64-column siblings
     (1000, 12700, 192), (300, 49000, 64), (2048, 6144, 4096),     # pipelined, 256 x 256 tiles
     (1000, 8200, 96), (130, 66000, 32), (2048, 4096, 4000),        # pipelined, 128 x 256 tiles
 ])
