@@ -913,6 +913,9 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
   }
   if (K % 32 == 0 && t128 >= lq_compute_units())
     return launch_pipelined<2, 2, 2, 4, 32, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+  // few tiles even of 128 x 256 (some hundred rows of a narrow matrix): 128 x 128 tiles, four stages deep
+  if (K % 64 == 0 && K >= 512)
+    return launch_pipelined<4, 2, 1, 2, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
   if (t128 >= 2 * lq_compute_units()) return launch_tiled<2, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   return launch_tiled<2, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
 }
