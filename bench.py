@@ -76,7 +76,9 @@ def main() -> int:
                     help="prompts of unequal lengths, uniform in [--prompt-len, this] (0 = all of --prompt-len)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (the headline run is 8b)")
     ap.add_argument("--no-points", action="store_true", help="skip the prefill and the batch 1 / 64 points")
-    ap.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
+    ap.add_argument("--prefill-only", action="store_true", help="run the prefill alone, twice (for profiling)")
+    ap.add_argument("--prefill-tokens", type=int, default=2048,
+                    help="prompt length of --prefill-only (the reported prefill is always of 2,048 tokens)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -131,15 +133,16 @@ def main() -> int:
         return batch * steps / dt, dt / steps * 1e3, ctx_mean
 
     if args.prefill_only:
+        n = args.prefill_tokens
         slot = engine.new_sequence()
-        engine.step([StepEntry(slot, random_prompt(2048), [2047])])
+        engine.step([StepEntry(slot, random_prompt(n), [n - 1])])
         engine.release(slot)
         slot = engine.new_sequence()
         torch.cuda.synchronize()
         t = time.perf_counter()
-        engine.step([StepEntry(slot, random_prompt(2048), [2047])])
+        engine.step([StepEntry(slot, random_prompt(n), [n - 1])])
         torch.cuda.synchronize()
-        print(f"[bench] prefill of 2048 tokens: {(time.perf_counter() - t) * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        print(f"[bench] prefill of {n} tokens: {(time.perf_counter() - t) * 1e3:.2f} ms", file=sys.stderr, flush=True)
         return 0
     value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
     step_bytes = weight_bytes_per_step(config) + args.batch * ctx_mean * kv_bytes_per_token(config)
@@ -152,16 +155,19 @@ def main() -> int:
         t_tokens = 2048
         slot = engine.new_sequence()
         prompt = random_prompt(t_tokens)
-        # once untimed (first launches), then timed on a fresh slot
+        # once untimed (first launches), then three times on fresh slots: the median
         engine.step([StepEntry(slot, prompt, [t_tokens - 1])])
         engine.release(slot)
-        slot = engine.new_sequence()
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        engine.step([StepEntry(slot, prompt, [t_tokens - 1])])
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t
-        engine.release(slot)
+        times = []
+        for _ in range(3):
+            slot = engine.new_sequence()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            engine.step([StepEntry(slot, prompt, [t_tokens - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            engine.release(slot)
+        dt = sorted(times)[1]
         prefill = {
             "value": round(t_tokens / dt, 1), "tokens": t_tokens, "ms": round(dt * 1e3, 3),
             "frac": round(prefill_flops(config, t_tokens) / dt / (BF16_TFLOPS * 1e12), 4),
