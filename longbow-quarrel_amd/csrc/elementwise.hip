@@ -81,7 +81,10 @@ __device__ inline void store4(bf16_t* p, f32x4_t v) {
   *(u32x2_t*)p = r;
 }
 
-template <typename TD, typename TO, bool HAS_DELTA, int NV>
+// MANY: the delta comes in more than two pieces (few rows of a product whose K many blocks share): such a
+// launch is bound by the latency of its loads, not by their number, and asks for four pieces of all of a
+// thread's elements together.  Many rows with one or two pieces stream, and want few registers instead.
+template <typename TD, typename TO, bool HAS_DELTA, int NV, bool MANY>
 __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ x, const TD* __restrict__ delta,
                                                            int parts, long long part_stride,
                                                            const float* __restrict__ w, TO* __restrict__ out,
@@ -90,16 +93,58 @@ __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ x
   const long long base = (long long)blockIdx.x * D;
   f32x4_t v[NV];
   float ss = 0.f;
+  if constexpr (!MANY) {
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int j = (threadIdx.x + i * 256) * 4;
-    if (j < D) {
-      v[i] = load4(x + base + j);
-      if (HAS_DELTA) {
-        for (int s = 0; s < parts; ++s) v[i] += load4(delta + s * part_stride + base + j);
-        store4(x + base + j, v[i]);
+    for (int i = 0; i < NV; ++i) {
+      const int j = (threadIdx.x + i * 256) * 4;
+      if (j < D) {
+        v[i] = load4(x + base + j);
+        if (HAS_DELTA) {
+          for (int s = 0; s < parts; ++s) v[i] += load4(delta + s * part_stride + base + j);
+          store4(x + base + j, v[i]);
+        }
+        ss += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
       }
-      ss += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int j = (threadIdx.x + i * 256) * 4;
+      if (j < D) v[i] = load4(x + base + j);
+    }
+    // the pieces are added in ascending order, element by element, as above
+    int s = 0;
+    for (; s + 4 <= parts; s += 4) {
+      f32x4_t d[4][NV];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const int j = (threadIdx.x + i * 256) * 4;
+          if (j < D) d[q][i] = load4(delta + (s + q) * part_stride + base + j);
+        }
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const int j = (threadIdx.x + i * 256) * 4;
+          if (j < D) v[i] += d[q][i];
+        }
+    }
+    for (; s < parts; ++s) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int j = (threadIdx.x + i * 256) * 4;
+        if (j < D) v[i] += load4(delta + s * part_stride + base + j);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int j = (threadIdx.x + i * 256) * 4;
+      if (j < D) {
+        store4(x + base + j, v[i]);
+        ss += v[i][0] * v[i][0] + v[i][1] * v[i][1] + v[i][2] * v[i][2] + v[i][3] * v[i][3];
+      }
     }
   }
   ss = block_sum(ss, red);
@@ -118,9 +163,15 @@ static void rmsnorm_launch(float* x, const void* delta, int parts, long long par
                        ((uintptr_t)w % 16) == 0 && ((uintptr_t)delta % 16) == 0 && part_stride % 4 == 0;
   const int vecs = (D / 4 + 255) / 256;
   if (aligned && vecs <= 8) {
-#define LQ_REGS(NV) \
-  rmsnorm_regs_kernel<TD, TO, HAS, NV><<<rows, 256, 0, stream>>>(x, (const TD*)delta, parts, part_stride, w, \
-                                                                 (TO*)out, D, eps)
+#define LQ_REGS(NV)                                                                                              \
+  do {                                                                                                           \
+    if (HAS && parts > 2)                                                                                        \
+      rmsnorm_regs_kernel<TD, TO, HAS, NV, true><<<rows, 256, 0, stream>>>(x, (const TD*)delta, parts,           \
+                                                                           part_stride, w, (TO*)out, D, eps);    \
+    else                                                                                                         \
+      rmsnorm_regs_kernel<TD, TO, HAS, NV, false><<<rows, 256, 0, stream>>>(x, (const TD*)delta, parts,          \
+                                                                            part_stride, w, (TO*)out, D, eps);   \
+  } while (0)
     if (vecs <= 1)
       LQ_REGS(1);
     else if (vecs <= 2)
@@ -262,8 +313,21 @@ __global__ void gather_rows_kernel(const float* __restrict__ x, const TD* __rest
   const long long dst = (long long)blockIdx.x * D;
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
     float v = x[src + j];
-    if (HAS_DELTA)
-      for (int s = 0; s < parts; ++s) v += to_f32(delta[s * part_stride + src + j]);
+    if (HAS_DELTA) {
+      // ascending order; four pieces are asked for together
+      int s = 0;
+      for (; s + 4 <= parts; s += 4) {
+        const float d0 = to_f32(delta[s * part_stride + src + j]);
+        const float d1 = to_f32(delta[(s + 1) * part_stride + src + j]);
+        const float d2 = to_f32(delta[(s + 2) * part_stride + src + j]);
+        const float d3 = to_f32(delta[(s + 3) * part_stride + src + j]);
+        v += d0;
+        v += d1;
+        v += d2;
+        v += d3;
+      }
+      for (; s < parts; ++s) v += to_f32(delta[s * part_stride + src + j]);
+    }
     out[dst + j] = v;
   }
 }
