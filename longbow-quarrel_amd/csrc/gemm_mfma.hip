@@ -11,7 +11,9 @@
 // Kernels:
 //  * tiled, pipelined: 4 or 8 waves compute a 128 x 256 or 256 x 256 tile; operand slabs go from
 //    memory straight into a ring of LDS stages (no registers in between).  For many rows (prefill)
-//    and K a multiple of 32.
+//    and K a multiple of 32.  The same kernel with tiles of 64, 128 or 256 rows by 128, 64 or 32
+//    columns and three or four stages takes 33 to 256 rows of a wide matrix (long decoding batches,
+//    short prompts): the tile covers all rows, so every weight is read once, at streaming speed.
 //  * tiled: a block of 4 waves (2 x 2) computes a (2*WM*32) x (2*WN*32) tile, operands staged
 //    through padded LDS in steps of 64 k, next step prefetched into registers while the current one
 //    is multiplied.  Takes any K that is a multiple of 8, and the small cases.
