@@ -266,6 +266,12 @@ def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory
     got = eng.step([StepEntry(s, long_prompt, range(300))])
     eng.release(s)
     assert rel_err(got, ref.forward(long_prompt, plain.round_bf16)) < TOL_BF16
+    # prompts of 33 to 256 rows: the pipelined tiles that cover all rows (64, 128 and 256 of them)
+    for n in (50, 100, 200):
+        s = eng.new_sequence()
+        got = eng.step([StepEntry(s, long_prompt[:n], range(n))])
+        eng.release(s)
+        assert rel_err(got, ref.forward(long_prompt[:n], plain.round_bf16)) < TOL_BF16
     # and inside a captured step
     g1 = lq.generate(eng, [r[:6] for r in reqs], 10, params=lq.SamplingParams(temperature=0.0), stop_ids=[], use_graphs=True)
     g2 = lq.generate(eng, [r[:6] for r in reqs], 10, params=lq.SamplingParams(temperature=0.0), stop_ids=[], use_graphs=False)
@@ -273,9 +279,10 @@ def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory
 
 
 def test_decoding_batches_that_shrink_from_40_rows_to_one(tmp_path_factory):
-    """40 sequences that end one after the other: decoding steps of 40 down to 1 row take the matrix-vector
-    kernels with four, two and one row tile (K shared between blocks, the pieces added by the norms; below
-    17 rows the norms folded into the products), against the plain implementation."""
+    """40 sequences that end one after the other: decoding steps of 40 down to 1 row take the pipelined
+    64-row tiles (above 32 rows), then the matrix-vector kernels with two and one row tile (K shared
+    between blocks, the pieces added by the norms; below 17 rows the norms folded into the products),
+    against the plain implementation."""
     folder = write_folder(tmp_path_factory.mktemp("wide64"), WIDE, seed=4, std=0.03)
     eng = lq.load_engine(folder, dtype="bfloat16", max_tokens=64 * 48)
     c, tensors = read_folder(folder)
