@@ -7,13 +7,13 @@ kernels.
 from . import models  # noqa: F401  (registers the architectures)
 from .api import QuarrelEngine, SamplerConfig, new_engine
 from .config import ConfigError, LlamaConfig, ModelConfig
-from .engine import Engine, GenerationResult, StepEntry, generate
+from .engine import Engine, GenerationResult, SequenceTooLong, StepEntry, generate
 from .loading import load_engine, random_engine
-from .sampling import SamplingParams
+from .sampling import NonFiniteLogits, SamplingParams
 from .registry import register_architecture, registered_architectures
 from .weights import WeightError, write_model_folder
 
 __all__ = [
     "ConfigError", "LlamaConfig", "ModelConfig", "Engine", "StepEntry", "load_engine", "random_engine",
-    "GenerationResult", "generate", "SamplingParams", "QuarrelEngine", "SamplerConfig", "new_engine", "register_architecture", "registered_architectures", "WeightError", "write_model_folder",
+    "GenerationResult", "generate", "SamplingParams", "NonFiniteLogits", "SequenceTooLong", "QuarrelEngine", "SamplerConfig", "new_engine", "register_architecture", "registered_architectures", "WeightError", "write_model_folder",
 ]

@@ -38,8 +38,11 @@ class SamplerConfig:
 class QuarrelEngine:
     def __init__(self, path: str, dtype: str = "bfloat16", kv_cache_size: int = 2048,
                  device: str = "cuda:0") -> None:
-        """`kv_cache_size`: tokens the cache holds (the reference's `KVCacheSize`, engine.go:388)."""
-        self.engine = load_engine(path, dtype=dtype, max_tokens=kv_cache_size, max_slots=1, device=device)
+        """`kv_cache_size`: tokens the cache holds (the reference's `KVCacheSize`, engine.go:388); an
+        explicit size is also the longest a sequence may get, whatever the configuration's context
+        length says (internal/engine/kv_cache_sliding_window.go:38-60)."""
+        self.engine = load_engine(path, dtype=dtype, max_tokens=kv_cache_size, max_slots=1, device=device,
+                                  max_sequence_tokens=kv_cache_size)
 
     def _run(self, tokens: Sequence[int], n: int, cfg: Optional[SamplerConfig],
              callback: Optional[Callable[[int], None]], keep_logits: bool) -> Tuple[List[int], Optional[torch.Tensor]]:
@@ -84,7 +87,7 @@ class QuarrelEngine:
         ids = torch.tensor([int(t) for t in tokens], dtype=torch.int32, device=e.device)
         out = torch.empty((len(tokens), self.embedding_dim()), dtype=torch.float32, device=e.device)
         if len(tokens):
-            e.run_on_stream(lambda: e.kernels.embed(e.model.embedding, ids, out))
+            e.run_on_stream(lambda: e.kernels.embed(e.model.embedding.table, ids, out))
         return out
 
     def get_embedding(self, token: int) -> torch.Tensor:

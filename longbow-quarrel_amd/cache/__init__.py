@@ -1,5 +1,5 @@
 """The cache: slots, paged keys and values per layer group, fixed-size state."""
-from .manager import CacheManager, KVGroup, StateGroup, blocks_for
+from .manager import CacheGroup, CacheManager, KVGroup, StateGroup, blocks_for
 from .slots import BLOCK_SIZE, CacheFull, FreeList
 
-__all__ = ["CacheManager", "KVGroup", "StateGroup", "blocks_for", "BLOCK_SIZE", "CacheFull", "FreeList"]
+__all__ = ["CacheGroup", "CacheManager", "KVGroup", "StateGroup", "blocks_for", "BLOCK_SIZE", "CacheFull", "FreeList"]

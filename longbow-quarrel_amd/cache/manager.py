@@ -2,7 +2,8 @@
 with each sequence's own length, and fixed-size state per sequence beside it.
 
 Layers are grouped by what their mixers need (`KVNeed`: kv heads, head size,
-window; `StateNeed`: a shape).  Every group has storage of its own: a pool of
+window; `StateNeed`: a shape; or a need class of the model's own).  Every need builds its
+group (`CacheNeed.make_group`) and every group has storage of its own: for keys and values a pool of
 blocks of BLOCK_SIZE positions and a block table per slot, so a group that keeps
 all positions and a group that keeps a window of them never share rows.  The
 reference has one contiguous ring per layer for its single sequence
@@ -20,7 +21,7 @@ from typing import Dict, List, Mapping, Optional, Tuple
 
 import torch
 
-from ..parts.base import KVNeed, LayerCache, StateNeed
+from ..parts.base import CacheNeed, KVNeed, LayerCache, StateNeed
 from .slots import BLOCK_SIZE, CacheFull, FreeList
 
 
@@ -28,7 +29,49 @@ def blocks_for(tokens: int) -> int:
     return (tokens + BLOCK_SIZE - 1) // BLOCK_SIZE
 
 
-class KVGroup:
+class CacheGroup:
+    """Storage of the runs of the schedule that share one need: what `CacheManager` asks of it.
+
+    A group that grows with a sequence's length takes blocks from a pool of its own and answers
+    `blocks_missing` / `free_blocks` / `blocks_for` truthfully, so that `CacheManager.reserve` can refuse
+    a step before anything has changed; a group of fixed size per slot keeps the defaults."""
+
+    layers: List[int]  # the runs of the schedule that the group serves
+
+    def layer_view(self, layer: int):
+        """What the mixer of run `layer` receives as `cache` (a `LayerCache`, or an object of the
+        group's own; it needs `read_only()` if another run may read it through `cache_of`)."""
+        raise NotImplementedError
+
+    def free_blocks(self) -> int:
+        """Blocks the pool can still hand out (a group without a pool: no limit)."""
+        return 1 << 60
+
+    def taken_blocks(self) -> int:
+        return 0
+
+    def blocks_for(self, tokens: int) -> int:
+        """Blocks a sequence of `tokens` tokens holds at most."""
+        return 0
+
+    def blocks_missing(self, slot: int, new_len: int) -> int:
+        """Blocks the slot still lacks for positions < new_len."""
+        return 0
+
+    def ensure(self, slot: int, new_len: int) -> None:
+        """Room for positions < new_len (the manager has checked `blocks_missing` against `free_blocks`)."""
+
+    def trim(self, slot: int, length: int) -> None:
+        """The slot holds `length` tokens now; what no later token can reach may go back."""
+
+    def release(self, slot: int) -> None:
+        """The sequence has ended: everything it holds goes back."""
+
+    def clear(self, slot: int) -> None:
+        """A new sequence starts in the slot."""
+
+
+class KVGroup(CacheGroup):
     """Storage of the layers that share one KVNeed."""
 
     def __init__(self, need: KVNeed, layers: List[int], n_blocks: int, max_slots: int,
@@ -54,6 +97,15 @@ class KVGroup:
         i = self.layers.index(layer)
         return LayerCache(write=True, k=self.k[i], v=self.v[i], block_table=self.table_dev,
                           block_size=BLOCK_SIZE)
+
+    def free_blocks(self) -> int:
+        return self.blocks.free_count
+
+    def taken_blocks(self) -> int:
+        return self.blocks.taken_count
+
+    def blocks_for(self, tokens: int) -> int:
+        return blocks_for(tokens)
 
     def blocks_missing(self, slot: int, new_len: int) -> int:
         return max(0, blocks_for(new_len) - len(self.owned[slot]))
@@ -90,7 +142,7 @@ class KVGroup:
         self.owned[slot] = []
 
 
-class StateGroup:
+class StateGroup(CacheGroup):
     """Fixed-size state of the layers that share one StateNeed: [layers, slots, *shape]."""
 
     def __init__(self, need: StateNeed, layers: List[int], max_slots: int, device: torch.device) -> None:
@@ -117,35 +169,39 @@ class CacheManager:
         self.max_slots = int(min(max_slots, self.n_blocks))
         self.slots = FreeList(self.max_slots, "slot")
         self.lengths = [0] * self.max_slots
-        self.kv_groups: List[KVGroup] = []
-        self.state_groups: List[StateGroup] = []
-        self._owner: Dict[int, object] = {}
+        self.groups: List[CacheGroup] = []
+        self._owner: Dict[int, CacheGroup] = {}
         by_need: Dict[object, List[int]] = {}
         for layer in sorted(needs):
             by_need.setdefault(needs[layer], []).append(layer)
         for need, layers in by_need.items():
-            if isinstance(need, KVNeed):
-                g = KVGroup(need, layers, self.n_blocks, self.max_slots, dtype, device)
-                self.kv_groups.append(g)
-            elif isinstance(need, StateNeed):
-                g = StateGroup(need, layers, self.max_slots, device)
-                self.state_groups.append(g)
-            else:
-                raise TypeError(f"layer {layers[0]}: unknown cache need {need!r}")
+            if not isinstance(need, CacheNeed):
+                raise TypeError(f"run {layers[0]} of the schedule: {need!r} is no CacheNeed "
+                                "(a need builds its own group: CacheNeed.make_group)")
+            g = need.make_group(layers, self.n_blocks, self.max_slots, dtype, device)
+            self.groups.append(g)
             for layer in layers:
                 self._owner[layer] = g
+
+    @property
+    def kv_groups(self) -> List[KVGroup]:
+        return [g for g in self.groups if isinstance(g, KVGroup)]
+
+    @property
+    def state_groups(self) -> List[StateGroup]:
+        return [g for g in self.groups if isinstance(g, StateGroup)]
 
     # ---- slots ------------------------------------------------------------------------
     def acquire(self) -> int:
         slot = self.slots.take()
         self.lengths[slot] = 0
-        for g in self.state_groups:
+        for g in self.groups:
             g.clear(slot)
         return slot
 
     def release(self, slot: int) -> None:
         self.slots.give(slot)  # raises if the slot is not in use
-        for g in self.kv_groups:
+        for g in self.groups:
             g.release(slot)
         self.lengths[slot] = 0
 
@@ -158,26 +214,34 @@ class CacheManager:
     def reserve(self, growth: Mapping[int, int]) -> None:
         """Makes room for `growth[slot]` more tokens in every slot named, or raises CacheFull
         before anything has changed."""
-        for g in self.kv_groups:
+        for g in self.groups:
             missing = sum(g.blocks_missing(slot, self.lengths[slot] + n) for slot, n in growth.items())
-            if missing > g.blocks.free_count:
+            if missing > g.free_blocks():
                 raise CacheFull(
                     f"the cache is full: {missing} more blocks of {BLOCK_SIZE} tokens are needed, "
-                    f"{g.blocks.free_count} of {g.n_blocks} are free")
-        for g in self.kv_groups:
+                    f"{g.free_blocks()} of {self.n_blocks} are free")
+        for g in self.groups:
             for slot, n in growth.items():
                 g.ensure(slot, self.lengths[slot] + n)
 
     def advance(self, growth: Mapping[int, int]) -> None:
         for slot, n in growth.items():
             self.lengths[slot] += n
-            for g in self.kv_groups:
+            for g in self.groups:
                 g.trim(slot, self.lengths[slot])
 
+    def free_blocks(self) -> int:
+        """Blocks that every group can still hand out."""
+        return min((g.free_blocks() for g in self.groups), default=1 << 60)
+
+    def blocks_for(self, tokens: int) -> int:
+        """Blocks a sequence of `tokens` tokens takes from the fullest-growing group."""
+        return max((g.blocks_for(tokens) for g in self.groups), default=0)
+
     # ---- views --------------------------------------------------------------------------------
-    def layer_views(self) -> Dict[int, LayerCache]:
+    def layer_views(self) -> Dict[int, object]:
         return {layer: g.layer_view(layer) for layer, g in self._owner.items()}
 
     def tokens_held(self) -> int:
         """Tokens of live sequences, each rounded up to whole blocks (largest over the groups)."""
-        return max((g.blocks.taken_count for g in self.kv_groups), default=0) * BLOCK_SIZE
+        return max((g.taken_blocks() for g in self.groups), default=0) * BLOCK_SIZE

@@ -69,9 +69,11 @@ def main(argv: Optional[List[str]] = None) -> int:
         with open(args.random_config) as f:
             from longbow_quarrel_amd.registry import config_from_dict
             config = config_from_dict(json.load(f))
-        engine = lq.random_engine(config, args.seed, dtype=args.dtype, max_tokens=max_tokens)
+        engine = lq.random_engine(config, args.seed, dtype=args.dtype, max_tokens=max_tokens,
+                                  max_sequence_tokens=args.kv_cache_size)
     else:
-        engine = lq.load_engine(args.model, dtype=args.dtype, max_tokens=max_tokens)
+        engine = lq.load_engine(args.model, dtype=args.dtype, max_tokens=max_tokens,
+                                max_sequence_tokens=args.kv_cache_size)
         tok_path = os.path.join(args.model, "tokenizer.json")
         if os.path.isfile(tok_path):
             from tokenizers import Tokenizer

@@ -924,26 +924,6 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
 
 }  // namespace
 
-// Tuning hook: one kernel, whatever the dispatcher would choose (float32 out, no epilogue).
-// (wm, wn) = (2, 2) or (2, 4): the register-staged kernel with that wave tile; wm = 0: a pipelined
-// kernel, wn = -1: 128 x 256 (4 waves, slabs of 32 k, 3 stages), -2: 256 x 256, -8: 256 x 192,
-// -9: 256 x 224 (8 waves, slabs of 64 k, 2 stages).
-extern "C" int lq_debug_gemm_tiled(const void* x, const void* w, void* out, int M, int N, int K, int wm, int wn,
-                                   hipStream_t stream) {
-  if (wm == 2 && wn == 2) return launch_tiled<2, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
-  if (wm == 2 && wn == 4) return launch_tiled<2, 4, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, stream);
-  if (wn == -1) return launch_pipelined<2, 2, 2, 4, 32, 3, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
-  if (wn == -2) return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
-  if (wn == -8) return launch_pipelined<4, 2, 2, 3, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
-  if (wn == -9) return launch_pipelined<8, 1, 1, 7, 64, 2, EPI_NONE, float>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
-  if (wn == -12)
-    return launch_pipelined<4, 2, 2, 4, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
-  if (wn == -13)
-    return launch_pipelined<4, 2, 2, 3, 64, 2, EPI_NONE, float, true>(x, w, out, M, N, K, K, K, N, 1, 0, stream);
-  lq_set_error("no such tile");
-  return -1;
-}
-
 int lq_gemm_mfma_splits(int M, int N, int K) { return mfma_splits(M, N, K); }
 
 // The decode pair around a norm.  `residual`: x[M, N] (float32) += act[M, K] . w[N, K]^T; sq_out[M][parts]

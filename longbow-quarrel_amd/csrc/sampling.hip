@@ -107,6 +107,20 @@ __device__ inline unsigned long long key_of(float logit, int index) {
   return ((unsigned long long)ordered_bits(logit) << 32) | (unsigned long long)(0xffffffffu - (unsigned)index);
 }
 
+// A row that holds a NaN or an infinity is not sampled from: its token comes out as NO_TOKEN, its
+// generator and ring stay as they are, and the host reports it (the reference scans the row the same
+// way and then takes the first finite index instead: internal/engine/sampler.go:72-75, 107-123).
+// BAD_ROW is larger than any key (the largest, of +inf at index 0, has 0xff800000 as its upper half).
+constexpr unsigned long long BAD_ROW = ~0ull;
+constexpr int NO_TOKEN = -1;
+
+__device__ inline bool non_finite(float f) { return (__float_as_uint(f) & 0x7f800000u) == 0x7f800000u; }
+
+// the key, or BAD_ROW for a NaN or an infinity
+__device__ inline unsigned long long checked_key_of(float logit, int index) {
+  return non_finite(logit) ? BAD_ROW : key_of(logit, index);
+}
+
 // splitmix64 of (key, counter): the n-th uniform of a sequence, 53 bits in [0, 1)
 __device__ inline double uniform_of(unsigned long long key, unsigned long long counter) {
   unsigned long long z = key + 0x9e3779b97f4a7c15ull * (counter + 1ull);
@@ -156,7 +170,7 @@ __global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restric
   const int i1 = min(V, (slice + 1) * per);
   unsigned long long best = 0ull;
   for (int i = slice * per + threadIdx.x; i < i1; i += 256) {
-    const unsigned long long k = key_of(lr[i], i);
+    const unsigned long long k = checked_key_of(lr[i], i);
     best = k > best ? k : best;
   }
   for (int off = 32; off > 0; off >>= 1) {
@@ -181,6 +195,10 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const unsigned long lo
     best = o > best ? o : best;
   }
   if (threadIdx.x == 0) {
+    if (best == BAD_ROW) {
+      out[row] = NO_TOKEN;
+      return;
+    }
     const int tok = (int)(0xffffffffu - (unsigned)(best & 0xffffffffull));
     out[row] = tok;
     if (recent) push_recent(recent, recent_n, seq_slot[row], tok);
@@ -400,10 +418,18 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a) {
   // maximum logit (as a key: also gives the arg-max)
   unsigned long long best = 0ull;
   for_each_logit(lr, V, [&](float v, int i) {
-    const unsigned long long k = key_of(v, i);
+    const unsigned long long k = checked_key_of(v, i);
     best = k > best ? k : best;
   });
   best = block_max_u64(best, smu);
+  if (best == BAD_ROW) {  // the same for every thread of the block
+    if (tid == 0) {
+      a.out[row] = NO_TOKEN;
+      if (a.kept_count) a.kept_count[row] = 0;
+      if (a.kept_mass) a.kept_mass[row] = 0.0;
+    }
+    return;
+  }
   const float mx = from_ordered_bits((unsigned)(best >> 32));
 
   // e_i = exp((l_i - max) / T) in 32-bit, sums in double; Z = sum e_i; candidates need p > 1e-10

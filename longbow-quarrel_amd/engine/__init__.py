@@ -1,5 +1,5 @@
 """The step function and the generation loop above it."""
 from .generate import EngineBackend, GenerationLoop, GenerationResult, generate
-from .step import Engine, StepEntry
+from .step import Engine, SequenceTooLong, StepEntry
 
-__all__ = ["Engine", "StepEntry", "EngineBackend", "GenerationLoop", "GenerationResult", "generate"]
+__all__ = ["Engine", "SequenceTooLong", "StepEntry", "EngineBackend", "GenerationLoop", "GenerationResult", "generate"]

@@ -8,11 +8,16 @@ kernel adds one to positions and lengths).  So the whole step (model, sampler,
 state upkeep) is captured once per batch size and replayed; the host only keeps
 the block tables ahead of the lengths and reads the sampled tokens back.
 
-A graph bakes in the pointers of its own workspace, logits buffer and integer
+A graph bakes in the pointers of the workspace, the logits buffer and its own integer
 arrays; the cache, the weights and the sampler state have fixed addresses for the
 life of the engine.  The split grid of the attention kernel depends on an upper
 bound of the lengths, so a graph is keyed by (B, bound) and a new one is captured
 when a sequence outgrows the bound.
+
+The graphs of one `DecodeGraphs` replay one at a time on one stream, so they share one
+workspace and one logits buffer, as large as the largest of them needs; when a new
+graph needs more than there is, the older graphs are dropped (their pointers would
+dangle) and captured again when their batch size comes back.
 """
 from __future__ import annotations
 
@@ -20,6 +25,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
+from ..kernels.dry import DryKernels
 from ..parts.base import StepContext, Workspace
 from ..sampling.sampler import Sampler
 
@@ -31,7 +37,7 @@ def _pad4(n: int) -> int:
 
 
 class DecodeGraph:
-    def __init__(self, engine, batch: int, bound: int) -> None:
+    def __init__(self, engine, batch: int, bound: int, ws: Workspace, logits: torch.Tensor) -> None:
         self.engine = engine
         self.batch = batch
         self.bound = bound
@@ -46,8 +52,8 @@ class DecodeGraph:
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=dev.type == "cuda")
         self.views = [self.meta[o : o + n] for o, n in zip(offs, self.sizes)]
         self.offs = offs
-        self.ws = Workspace(dev, 1 << 16)
-        self.logits = torch.empty((batch, engine.vocab_size), dtype=torch.float32, device=dev)
+        self.ws = ws
+        self.logits = logits  # [batch, vocab], rows of the shared buffer
         self.handle: Optional[int] = None
         self.slots: List[int] = []
 
@@ -67,14 +73,11 @@ class DecodeGraph:
         self.meta.copy_(h)
         self.slots = list(slots)
 
-    def context(self) -> StepContext:
+    def context(self, dry: bool = False) -> StepContext:
         e = self.engine
-        t, row_seq, row_pos, slot, start, length, cu, _want = self.views
-        return StepContext(
-            kernels=e.kernels, dtype=e.dtype, device=e.device, ws=self.ws, rows=self.batch, batch=self.batch,
-            tokens=t, row_seq=row_seq, row_pos=row_pos, seq_slot=slot, seq_start=start, seq_len=length,
-            cu_rows=cu, host_slots=list(self.slots), host_start=[], host_new=[1] * self.batch,
-            max_new=1, max_len=self.bound, decode=True, logits_out=self.logits)
+        return e.make_context(self.ws, self.views[:7], self.slots or [0] * self.batch, [], [1] * self.batch,
+                              self.bound, logits_out=self.logits,
+                              kernels=DryKernels(e.kernels) if dry else None, dry=dry)
 
     def run_body(self, sampler: Sampler) -> None:
         """What one decoding step launches; the same calls whether captured or run directly."""
@@ -85,37 +88,21 @@ class DecodeGraph:
         sampler.sample(self.logits, self.views[3], self.views[0])
         e.kernels.advance(self.views[2], self.views[4], self.views[5], self.batch)
 
+    def walk(self) -> bool:
+        """Walks through the body's allocations without launching (the workspace must not be frozen:
+        what does not fit comes from the allocator for the walk); False if the workspace was too small."""
+        e = self.engine
+        self.ws.reset()
+        e.model.forward(self.context(dry=True), e.cache.layer_views(), self.views[7], self.batch)
+        return self.ws.fits()
+
     def capture(self, sampler: Sampler) -> None:
         kn = self.engine.kernels
-        # a dry pass sizes the workspace (captures must not allocate)
-        self._size_workspace(sampler)
         kn.graph_begin()
         try:
             self.run_body(sampler)
         finally:
             self.handle = kn.graph_end()
-        self.ws.frozen = True
-
-    def _size_workspace(self, sampler: Sampler) -> None:
-        """Runs the body's allocations without launching, to learn the workspace size."""
-        e = self.engine
-
-        queries = ("attention_workspace", "attention_folds_rope", "linear_swiglu_supported", "linear_pieces",
-                   "linear_fused_parts")
-
-        class _Null:
-            """Answers the size and capability questions truthfully, launches nothing."""
-
-            def __getattr__(self, name):
-                if name in queries:
-                    return getattr(e.kernels, name)
-                return lambda *a, **k: None
-
-        ctx = self.context()
-        ctx.kernels = _Null()
-        self.ws.reset()
-        e.model.forward(ctx, e.cache.layer_views(), self.views[7], self.batch)
-        self.ws.reset()  # grows the buffer to the high-water mark
 
     def launch(self) -> None:
         self.engine.kernels.graph_launch(self.handle)
@@ -124,3 +111,48 @@ class DecodeGraph:
         if self.handle is not None:
             self.engine.kernels.graph_destroy(self.handle)
             self.handle = None
+
+
+class DecodeGraphs:
+    """The captured decoding steps of one backend, keyed by (batch size, length bound), and the
+    workspace and logits buffer that they share."""
+
+    graph_cls = DecodeGraph
+
+    def __init__(self, engine, sampler: Sampler) -> None:
+        self.engine = engine
+        self.sampler = sampler
+        self.ws = Workspace(engine.device, 1 << 16)
+        self.logits: Optional[torch.Tensor] = None
+        self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}
+        self.captures = 0
+
+    def get(self, batch: int, bound: int) -> Tuple[DecodeGraph, bool]:
+        """The graph for this batch size and bound, and whether it is new (then the caller loads its
+        arrays and calls `capture`)."""
+        key = (batch, bound)
+        g = self.graphs.get(key)
+        if g is not None:
+            return g, False
+        e = self.engine
+        if self.logits is None or self.logits.shape[0] < batch:
+            self.drop_all()
+            self.logits = torch.empty((batch, e.vocab_size), dtype=torch.float32, device=e.device)
+        g = self.graph_cls(e, batch, bound, self.ws, self.logits[:batch])
+        self.ws.frozen = False
+        if not g.walk():
+            self.drop_all()  # the buffers are about to move: the graphs that point into them go
+        self.ws.reset()  # grows the buffers to what the walk needed
+        self.ws.frozen = True
+        self.graphs[key] = g
+        self.captures += 1
+        return g, True
+
+    def drop_all(self) -> None:
+        for g in self.graphs.values():
+            g.destroy()
+        self.graphs.clear()
+        self.ws.frozen = False
+
+    def close(self) -> None:
+        self.drop_all()

@@ -13,9 +13,12 @@ its habits are not kept: the stop id is hard-coded and the first sampled token i
 never checked against it (:1744-1747); here stop ids come from the configuration
 or the caller and every sampled token is checked.
 
-`GenerationLoop` holds the decisions only and talks to a backend with five
+`GenerationLoop` holds the decisions only and talks to a backend with a handful of
 methods, so that the decisions can be tested without a GPU; `EngineBackend` is the
-real one.
+real one.  It feeds a batch's prompts in portions of at most `max_prefill_rows` rows
+(the step's workspace grows with its rows, not with the batch), and it reports a row of
+logits that holds a NaN or an infinity as `NonFiniteLogits` where the reference takes
+the first finite index (internal/engine/sampler.go:72-75, 107-123).
 """
 from __future__ import annotations
 
@@ -27,10 +30,10 @@ import torch
 
 from ..cache import BLOCK_SIZE, CacheFull
 from ..sampling.params import SamplingParams
-from ..sampling.sampler import Sampler
+from ..sampling.sampler import NonFiniteLogits, Sampler
 from ..sampling.state import SamplerState, sequence_key
-from .decode import LEN_BUCKET, DecodeGraph
-from .step import Engine, StepEntry
+from .decode import LEN_BUCKET, DecodeGraphs
+from .step import Engine, SequenceTooLong, StepEntry
 
 
 @dataclass
@@ -53,12 +56,12 @@ class GenerationLoop:
         self.backend = backend
         self.max_batch = max_batch
 
-    def _next_batch(self, pending: List[int], prompts: Sequence[Sequence[int]], max_new: int) -> List[int]:
+    def _next_batch(self, pending: List[int], prompts: Sequence[Sequence[int]], limit: Sequence[int]) -> List[int]:
         """The longest prefix of the pending requests that fits the batch size and the cache."""
         budget = self.backend.free_blocks()
         chosen: List[int] = []
         for r in pending:
-            need = self.backend.blocks_needed(len(prompts[r]) + max_new)
+            need = self.backend.blocks_needed(len(prompts[r]) + limit[r])
             if len(chosen) >= self.max_batch or need > budget:
                 break
             chosen.append(r)
@@ -66,8 +69,21 @@ class GenerationLoop:
         if not chosen:
             r = pending[0]
             raise CacheFull(
-                f"request {r} needs room for {len(prompts[r]) + max_new} tokens, more than the cache can hold")
+                f"request {r} needs room for {len(prompts[r]) + limit[r]} tokens, more than the cache can hold")
         return chosen
+
+    def _token_limits(self, prompts: Sequence[Sequence[int]], max_new_tokens: int) -> List[int]:
+        """How many tokens each request may get: `max_new_tokens`, or fewer where the sequence would
+        pass the length a sequence may have (the last sampled token is never fed back, so a sequence
+        that holds n tokens has produced n - prompt + 1)."""
+        room = getattr(self.backend, "token_room", None)
+        limits = []
+        for r, p in enumerate(prompts):
+            k = room(len(p)) if room is not None else None
+            if k is not None and k <= 0:
+                raise SequenceTooLong(f"request {r}: its prompt of {len(p)} tokens is longer than a sequence may be")
+            limits.append(max_new_tokens if k is None else min(max_new_tokens, k))
+        return limits
 
     def run(self, prompts: Sequence[Sequence[int]], max_new_tokens: int, stop_ids: Sequence[int] = (),
             include_stop: bool = False, callback: Optional[Callable[[int, int], None]] = None) -> GenerationResult:
@@ -79,10 +95,11 @@ class GenerationLoop:
         result = GenerationResult(tokens=[[] for _ in range(n)], finish=["length"] * n)
         if max_new_tokens <= 0 or n == 0:
             return result
+        limit = self._token_limits(prompts, max_new_tokens)
         pending = list(range(n))
         be = self.backend
         while pending:
-            batch = self._next_batch(pending, prompts, max_new_tokens)
+            batch = self._next_batch(pending, prompts, limit)
             pending = pending[len(batch):]
             result.batches += 1
             slots: Dict[int, int] = {}
@@ -94,6 +111,7 @@ class GenerationLoop:
                 result.prefill_seconds += time.perf_counter() - t0
                 result.prefill_tokens += sum(len(prompts[r]) for r in batch)
                 live = list(batch)
+                first = True  # a batch's first decoding step always brings new sequences
                 t0 = time.perf_counter()
                 while True:
                     survivors: List[int] = []
@@ -110,14 +128,15 @@ class GenerationLoop:
                         result.tokens[r].append(tok)
                         if callback:
                             callback(r, tok)
-                        if len(result.tokens[r]) >= max_new_tokens:
+                        if len(result.tokens[r]) >= limit[r]:
                             result.finish[r] = "length"
                             be.release(slots.pop(r))
                             continue
                         survivors.append(r)
                     if not survivors:
                         break
-                    changed = survivors != live
+                    changed = first or survivors != live
+                    first = False
                     live = survivors
                     sampled = be.decode([slots[r] for r in live],
                                         [result.tokens[r][-1] for r in live], changed)
@@ -133,36 +152,80 @@ class EngineBackend:
     """Drives an `Engine` for the loop: prompts through `Engine.step`, single-token steps through
     captured graphs (or through `Engine.step` when graphs are off), sampling on the device."""
 
-    def __init__(self, engine: Engine, params: SamplingParams, use_graphs: bool = True) -> None:
+    def __init__(self, engine: Engine, params: SamplingParams, use_graphs: bool = True,
+                 max_prefill_rows: int = 8192, graphs_cls=DecodeGraphs) -> None:
+        if max_prefill_rows <= 0:
+            raise ValueError("max_prefill_rows must be positive")
         self.engine = engine
         self.params = params
+        self.max_prefill_rows = int(max_prefill_rows)
         if not hasattr(engine, "sampler_state"):
             engine.sampler_state = SamplerState(engine.cache.max_slots, engine.device)
         self.sampler = Sampler(engine.kernels, engine.sampler_state, params)
-        self.use_graphs = use_graphs and engine.device.type == "cuda" and engine.graph_safe
-        self.graphs: Dict[tuple, DecodeGraph] = {}
-        self.current: Optional[DecodeGraph] = None
-        self.keep_logits = False  # direct steps only: a copy of each step's logits before sampling changes them
+        self.use_graphs = use_graphs and engine.graph_safe and \
+            (engine.device.type == "cuda" or graphs_cls is not DecodeGraphs)
+        self.graphs = graphs_cls(engine, self.sampler) if self.use_graphs else None
+        self.current = None  # the graph whose arrays hold the live batch, as the last step left them
+        self.request_of: Dict[int, int] = {}  # slot -> index of the request that runs there
+        # a copy of each step's logits: before sampling where steps run directly, as the sampler left them
+        # (with the repetition penalty applied, if there is one) where they are replayed from a graph
+        self.keep_logits = False
         self.last_logits: Optional[torch.Tensor] = None
+        self.prefill_steps = 0
 
     # ---- what the loop asks ------------------------------------------------------------
     def free_blocks(self) -> int:
-        return min((g.blocks.free_count for g in self.engine.cache.kv_groups), default=1 << 30)
+        return self.engine.cache.free_blocks()
 
     def blocks_needed(self, tokens: int) -> int:
-        return (tokens + BLOCK_SIZE - 1) // BLOCK_SIZE
+        return self.engine.cache.blocks_for(tokens)
+
+    def token_room(self, prompt_tokens: int) -> Optional[int]:
+        """How many tokens a request with such a prompt can get before its sequence is as long as
+        one may be (None: no bound)."""
+        limit = self.engine.max_sequence_tokens
+        return None if limit is None else limit - prompt_tokens + 1
 
     def new_sequence(self, request_index: int, prompt: Sequence[int]) -> int:
         slot = self.engine.new_sequence()
         self.engine.sampler_state.start(slot, sequence_key(self.params.seed, request_index), prompt)
+        self.request_of[slot] = request_index
+        self.current = None  # whatever a graph's arrays hold is of an earlier batch
         return slot
 
     def release(self, slot: int) -> None:
+        self.request_of.pop(slot, None)
         self.engine.release(slot)
 
     def prefill(self, slots: Sequence[int], prompts: Sequence[Sequence[int]]) -> List[int]:
+        """Runs the prompts, in as many steps as `max_prefill_rows` asks for (a step takes the next
+        tokens of as many sequences as fit, a long prompt goes on in the next step), and samples each
+        sequence's first token from the logits at its last place."""
         e = self.engine
-        logits = e.step([StepEntry(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])
+        self.current = None
+        rows_out: List[Optional[torch.Tensor]] = [None] * len(slots)
+        at = [0] * len(slots)  # tokens of each prompt that have run
+        steps = 0
+        i = 0
+        while i < len(slots):
+            entries, owners, room = [], [], self.max_prefill_rows
+            while i < len(slots) and room > 0:
+                n = min(room, len(prompts[i]) - at[i])
+                last = at[i] + n == len(prompts[i])
+                entries.append(StepEntry(slots[i], prompts[i][at[i] : at[i] + n], [n - 1] if last else []))
+                at[i] += n
+                room -= n
+                if not last:
+                    break  # the step is full; this prompt goes on in the next one
+                owners.append(i)
+                i += 1
+            logits = e.step(entries)
+            steps += 1
+            for k, owner in enumerate(owners):
+                rows_out[owner] = logits[k : k + 1]
+        self.prefill_steps += steps
+        if steps > 1:
+            logits = torch.cat(rows_out)  # each sequence's row, side by side for the sampler
         return self._sample_eager(logits, slots)
 
     def decode(self, slots: Sequence[int], last_tokens: Sequence[int], changed: bool) -> List[int]:
@@ -173,6 +236,14 @@ class EngineBackend:
         return e.run_on_stream(lambda: self._decode_graph(list(slots), list(last_tokens), changed))
 
     # ---- internals ------------------------------------------------------------------------
+    def _checked(self, tokens: List[int], slots: Sequence[int]) -> List[int]:
+        """The sampler's answer for a row of logits with a NaN or an infinity is no token."""
+        bad = [s for s, t in zip(slots, tokens) if t < 0]
+        if bad:
+            names = ", ".join(f"request {self.request_of.get(s, '?')} (slot {s})" for s in bad)
+            raise NonFiniteLogits(f"the logits of {names} hold a NaN or an infinity; nothing was sampled from them")
+        return tokens
+
     def _sample_eager(self, logits: torch.Tensor, slots: Sequence[int]) -> List[int]:
         e = self.engine
 
@@ -184,22 +255,21 @@ class EngineBackend:
             self.sampler.sample(logits, seq_slot, out)
             return out.cpu().tolist()
 
-        return e.run_on_stream(body)
+        return self._checked(e.run_on_stream(body), slots)
 
     def _decode_graph(self, slots: List[int], last_tokens: List[int], changed: bool) -> List[int]:
         e = self.engine
         cache = e.cache
         starts = [cache.length(s) for s in slots]
+        for s, n in zip(slots, starts):
+            e.check_room(s, n, 1)
         growth = {s: 1 for s in slots}
         cache.reserve(growth)
         longest = max(starts) + 1
         bound = (longest + LEN_BUCKET - 1) // LEN_BUCKET * LEN_BUCKET
-        key = (len(slots), bound)
-        g = self.graphs.get(key)
-        fresh = g is None
-        if fresh:
-            g = DecodeGraph(e, len(slots), bound)
-            self.graphs[key] = g
+        g, fresh = self.graphs.get(len(slots), bound)
+        # a graph's arrays carry on from its own last step only: anything else in between (another graph,
+        # a prompt step, a batch whose members changed) means they are written anew
         if fresh or changed or g is not self.current or g.slots != slots:
             g.load(slots, last_tokens, starts)
         if fresh:
@@ -208,24 +278,29 @@ class EngineBackend:
         g.launch()
         cache.advance(growth)
         e.steps_run += 1
-        return g.views[0].cpu().tolist()
+        if self.keep_logits:
+            self.last_logits = g.logits.clone()
+        return self._checked(g.views[0].cpu().tolist(), slots)
 
     def close(self) -> None:
-        for g in self.graphs.values():
-            g.destroy()
-        self.graphs.clear()
+        if self.graphs is not None:
+            self.graphs.close()
+        self.current = None
 
 
 def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: int,
              params: Optional[SamplingParams] = None, stop_ids: Optional[Sequence[int]] = None,
              include_stop: bool = False, max_batch: int = 64, use_graphs: bool = True,
-             callback: Optional[Callable[[int, int], None]] = None) -> GenerationResult:
+             callback: Optional[Callable[[int, int], None]] = None, max_prefill_rows: int = 8192,
+             extra_stop_ids: Sequence[int] = ()) -> GenerationResult:
     """Generates up to `max_new_tokens` ids for every prompt.  `stop_ids` defaults to the
-    configuration's end-of-sequence ids."""
+    configuration's end-of-sequence ids (an explicit list stands in their place; `extra_stop_ids`
+    are added to whichever it is)."""
     params = params or SamplingParams()
     if stop_ids is None:
         stop_ids = tuple(engine.model.spec.stop_ids)
-    backend = EngineBackend(engine, params, use_graphs=use_graphs)
+    stop_ids = tuple(stop_ids) + tuple(extra_stop_ids)
+    backend = EngineBackend(engine, params, use_graphs=use_graphs, max_prefill_rows=max_prefill_rows)
     try:
         return GenerationLoop(backend, max_batch=max_batch).run(prompts, max_new_tokens, stop_ids,
                                                                 include_stop, callback)

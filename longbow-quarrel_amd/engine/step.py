@@ -10,7 +10,11 @@ position n + r, writes its key and value first and then attends to positions
 generalised from one sequence to a batch.
 
 The reference validates its input the same way (empty input, ids outside the
-vocabulary: internal/engine/engine.go:1300-1331).
+vocabulary: internal/engine/engine.go:1300-1331), and refuses a position at or past
+the length its cache was made for (internal/engine/kv_cache.go:121-124); here that
+length is `max_sequence_tokens`: the caller's explicit figure if there is one, else
+what the configuration allows (the reference sizes its cache in that order too:
+internal/engine/kv_cache_sliding_window.go:38-60).
 """
 from __future__ import annotations
 
@@ -22,6 +26,10 @@ import torch
 from ..cache import CacheManager
 from ..model import DecoderModel
 from ..parts.base import BuildEnv, StepContext, Workspace
+
+
+class SequenceTooLong(ValueError):
+    """A step would take a sequence past `Engine.max_sequence_tokens`."""
 
 
 @dataclass
@@ -70,7 +78,10 @@ class StepMeta:
 class Engine:
     """A model bound to a device, its cache and its step function."""
 
-    def __init__(self, model: DecoderModel, env: BuildEnv, max_tokens: int, max_slots: int = 256) -> None:
+    def __init__(self, model: DecoderModel, env: BuildEnv, max_tokens: int, max_slots: int = 256,
+                 max_sequence_tokens: Optional[int] = None) -> None:
+        """`max_tokens` sizes the cache's pool (all live sequences together); `max_sequence_tokens` bounds
+        one sequence (default: the longest the model's configuration allows; None there: the pool)."""
         self.model = model
         self.env = env
         self.kernels = env.kernels
@@ -78,12 +89,17 @@ class Engine:
         self.dtype = env.dtype
         self.vocab_size = model.spec.vocab_size
         self.cache = CacheManager(model.cache_needs(), max_tokens, max_slots, env.dtype, env.device)
+        if max_sequence_tokens is None:
+            max_sequence_tokens = model.spec.max_positions
+        if max_sequence_tokens is not None and max_sequence_tokens <= 0:
+            raise ValueError(f"max_sequence_tokens must be positive, found {max_sequence_tokens}")
+        self.max_sequence_tokens: Optional[int] = max_sequence_tokens
         self.ws = Workspace(env.device)
         self.meta = StepMeta(env.device)
         self.stream = torch.cuda.Stream(device=env.device) if env.device.type == "cuda" else None
         self.steps_run = 0
         #: whether every part only launches library kernels (then decoding steps can be captured)
-        self.graph_safe = all(getattr(b, "graph_safe", False) for b in model.blocks)
+        self.graph_safe = model.graph_safe
 
     # ---- sequences ---------------------------------------------------------------------
     def new_sequence(self) -> int:
@@ -106,15 +122,22 @@ class Engine:
             if e.slot in seen:
                 raise ValueError(f"slot {e.slot} appears twice in one step")
             seen.add(e.slot)
-            self.cache.length(e.slot)  # raises if the slot is not in use
+            held = self.cache.length(e.slot)  # raises if the slot is not in use
             if len(e.tokens) == 0:
                 raise ValueError(f"slot {e.slot}: a step entry needs at least one token")
+            self.check_room(e.slot, held, len(e.tokens))
             for t in e.tokens:
                 if not 0 <= int(t) < self.vocab_size:
                     raise ValueError(f"slot {e.slot}: token id {t} is outside the vocabulary [0, {self.vocab_size})")
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"slot {e.slot}: wanted place {w} is outside its {len(e.tokens)} tokens")
+
+    def check_room(self, slot: int, held: int, new: int) -> None:
+        limit = self.max_sequence_tokens
+        if limit is not None and held + new > limit:
+            raise SequenceTooLong(f"slot {slot}: {held} tokens held and {new} more would pass the "
+                                  f"{limit} tokens a sequence may have (max_sequence_tokens)")
 
     def run_on_stream(self, fn):
         """Runs fn() with the engine's stream current, ordered after what the caller has queued and
@@ -137,6 +160,22 @@ class Engine:
         debugging, sees the residual stream after the embedding and after every run of the schedule."""
         self._validate(entries)
         return self.run_on_stream(lambda: self._step(entries, observe))
+
+    def make_context(self, ws: Workspace, arrays: Sequence[torch.Tensor], slots: Sequence[int],
+                     starts: Sequence[int], new: Sequence[int], max_len: int, logits_out=None, observe=None,
+                     kernels=None, dry: bool = False) -> StepContext:
+        """The one place where a step's `StepContext` is put together, for direct and for captured steps.
+        `arrays`: the device arrays tokens, row_seq, row_pos, seq_slot, seq_start, seq_len, cu_rows;
+        `slots`, `starts`, `new`: per sequence, on the host (`starts` may be empty where the lengths
+        live on the device only, as in a captured step); `max_len`: an upper bound of the lengths after
+        the step."""
+        tokens, row_seq, row_pos, seq_slot, seq_start, seq_len, cu_rows = arrays
+        return StepContext(
+            kernels=kernels if kernels is not None else self.kernels, dtype=self.dtype, device=self.device, ws=ws,
+            rows=sum(new), batch=len(new), tokens=tokens, row_seq=row_seq, row_pos=row_pos, seq_slot=seq_slot,
+            seq_start=seq_start, seq_len=seq_len, cu_rows=cu_rows, host_slots=list(slots), host_start=list(starts),
+            host_new=list(new), max_new=max(new), max_len=max_len, decode=all(n == 1 for n in new),
+            logits_out=logits_out, observe=observe, dry=dry)
 
     def _step(self, entries: Sequence[StepEntry], observe=None) -> Optional[torch.Tensor]:
         cache = self.cache
@@ -164,14 +203,8 @@ class Engine:
             [tokens, row_seq, row_pos, slots, starts, lens, cu, want_rows])
 
         self.ws.reset()
-        ctx = StepContext(
-            kernels=self.kernels, dtype=self.dtype, device=self.device, ws=self.ws,
-            rows=len(tokens), batch=len(entries), tokens=d_tokens, row_seq=d_row_seq, row_pos=d_row_pos,
-            seq_slot=d_slot, seq_start=d_start, seq_len=d_len, cu_rows=d_cu,
-            host_slots=slots, host_start=starts, host_new=[len(e.tokens) for e in entries],
-            max_new=max(len(e.tokens) for e in entries), max_len=max(lens),
-            decode=all(len(e.tokens) == 1 for e in entries), observe=observe,
-        )
+        ctx = self.make_context(self.ws, (d_tokens, d_row_seq, d_row_pos, d_slot, d_start, d_len, d_cu), slots,
+                                starts, [len(e.tokens) for e in entries], max(lens), observe=observe)
         logits = self.model.forward(ctx, cache.layer_views(), d_want, len(want_rows))
         cache.advance(growth)
         self.steps_run += 1

@@ -17,6 +17,7 @@ from typing import Optional
 import torch
 
 from .. import build as _build
+from .dry import query
 
 F32, BF16 = 0, 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -168,6 +169,7 @@ class HipKernels:
         self._check(self.lib.lq_cast(_ptr(src), c_int(_code(src)), _ptr(out), c_int(_code(out)),
                                      c_longlong(src.numel()), self.stream))
 
+    @query
     def linear_pieces(self, dtype: torch.dtype, m: int, n: int, k: int) -> int:
         """In how many pieces `linear` would like to leave this product (1: whole).  A caller whose
         consumer adds pieces (`rmsnorm`, `add`, `gather_rows` with a stacked delta) may pass an output
@@ -204,6 +206,7 @@ class HipKernels:
 
     # -- the two products around a norm, for a few rows (decoding): x += act . w^T leaves every row's
     # sum of squares in parts, and the product after the norm normalises its input from them itself
+    @query
     def linear_fused_parts(self, dtype: torch.dtype, m: int, n: int, k: int) -> int:
         """How many parts `linear_residual` leaves a row for [m, k] x [n, k]^T; 0: these kernels do
         not take the size (use `linear` and `rmsnorm`)."""
@@ -254,6 +257,7 @@ class HipKernels:
                                               c_int(self._rows2d(w, "w")), c_int(self._rows2d(out, "out")),
                                               c_int(1 if swiglu else 0), self.stream))
 
+    @query
     def linear_swiglu_supported(self, dtype: torch.dtype, rows_out: int, k: int) -> bool:
         """Whether `linear_swiglu` takes weights of this dtype with `rows_out` (= 2 I) rows and width k."""
         if self.force_generic or dtype not in _DTYPE_CODE:
@@ -353,6 +357,7 @@ class HipKernels:
             _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(block_table), c_int(bt_stride),
             _ptr(kcache), _ptr(vcache), c_int(block_size), c_int(1 if store else 0), self.stream))
 
+    @query
     def attention_workspace(self, dtype: torch.dtype, rows: int, heads: int, kv_heads: int, head_dim: int,
                             block_size: int, decode: bool, max_len: int) -> int:
         """Float32 entries of scratch that `attention` wants for this launch (0: none)."""
@@ -363,6 +368,7 @@ class HipKernels:
                                                    c_int(kv_heads), c_int(head_dim), c_int(block_size),
                                                    c_int(1 if decode else 0), c_int(max_len)))
 
+    @query
     def attention_folds_rope(self, dtype: torch.dtype, heads: int, kv_heads: int, head_dim: int, block_size: int) -> bool:
         """Whether a decoding `attention` launch can rotate q and k and write the cache itself."""
         if self.force_generic or dtype not in _DTYPE_CODE:
@@ -428,7 +434,7 @@ class HipKernels:
             if cos_sin.dtype != torch.float32 or tuple(cos_sin.shape) != (rows, head_dim // 2, 2) or not cos_sin.is_contiguous():
                 raise KernelLibraryError("attention: cos_sin must be dense float32 [rows, head_dim/2, 2]")
             ldk, ldv = self._rows2d(k_new, "k_new"), self._rows2d(v_new, "v_new")
-        self._check(self.lib.lq_attention(
+        rc = self.lib.lq_attention(
             _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")),
             c_int(_code(q)), c_int(rows), c_int(batch), c_int(heads), c_int(kv_heads), c_int(head_dim),
             _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(cu_rows), _ptr(block_table),
@@ -436,7 +442,16 @@ class HipKernels:
             c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
             c_longlong(ws_n), _ptr(self._tickets), c_longlong(self._tickets.numel()), _ptr(k_new if cos_sin is not None else None),
             _ptr(v_new if cos_sin is not None else None), c_int(ldk), c_int(ldv), _ptr(cos_sin),
-            c_int(1 if self.force_generic else 0), self.stream))
+            c_int(1 if self.force_generic else 0), self.stream)
+        if rc != 0:
+            # a launch that did not run whole may have left tickets behind, and a later launch that found
+            # them non-zero would never recognise its last workgroup: clear them (a fill kernel) before
+            # the error goes up
+            message = self.lib.lq_last_error().decode("utf-8", "replace")
+            try:
+                self._tickets.zero_()
+            finally:
+                raise KernelLibraryError(message)
 
     # ------------------------------------------------------------------ sampling
     def apply_penalty(self, logits: torch.Tensor, seq_slot: torch.Tensor, recent: torch.Tensor,

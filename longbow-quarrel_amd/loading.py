@@ -40,14 +40,16 @@ def _env(dtype, device, kernels) -> BuildEnv:
 
 def load_engine(folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_tokens: int = 8192,
                 max_slots: int = 256, device: Union[str, torch.device] = "cuda:0",
-                kernels: Any = None) -> Engine:
-    """config.json chooses the model class; model.safetensors is bound by tensor name."""
+                kernels: Any = None, max_sequence_tokens: Optional[int] = None) -> Engine:
+    """config.json chooses the model class; model.safetensors is bound by tensor name.
+    `max_tokens` sizes the cache for all live sequences together; `max_sequence_tokens` bounds one
+    sequence (default: what the configuration allows, `max_position_embeddings` for Llama)."""
     config = config_from_dict(read_config_json(folder))
     model = DecoderModel(spec_from_config(config))
     env = _env(dtype, device, kernels)
     tensors = load_tensors(folder, model.tensor_specs(), env.dtype, env.device)
     model.bind(tensors, env)
-    engine = Engine(model, env, max_tokens, max_slots)
+    engine = Engine(model, env, max_tokens, max_slots, max_sequence_tokens)
     engine.config = config
     return engine
 
@@ -55,7 +57,7 @@ def load_engine(folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_to
 def random_engine(config: ModelConfig, seed: int, dtype: Union[str, torch.dtype] = "bfloat16",
                   max_tokens: int = 8192, max_slots: int = 256,
                   device: Union[str, torch.device] = "cuda:0", kernels: Any = None,
-                  std: float = 0.02) -> Engine:
+                  std: float = 0.02, max_sequence_tokens: Optional[int] = None) -> Engine:
     """Random weights made in memory on the device (nothing is written)."""
     model = DecoderModel(spec_from_config(config))
     env = _env(dtype, device, kernels)
@@ -66,6 +68,6 @@ def random_engine(config: ModelConfig, seed: int, dtype: Union[str, torch.dtype]
             tensors[s.name] = tensors[s.name].float()
     check_names_and_shapes(specs, {n: tuple(t.shape) for n, t in tensors.items()}, "random weights")
     model.bind(tensors, env)
-    engine = Engine(model, env, max_tokens, max_slots)
+    engine = Engine(model, env, max_tokens, max_slots, max_sequence_tokens)
     engine.config = config
     return engine

@@ -1,7 +1,8 @@
 """A decoder model as data (`ModelSpec`) and the object built from it.
 
-`ModelSpec` names the token embedding, the layers (each a block spec), the
-order in which layers run, the final norm and the output head.  `DecoderModel`
+`ModelSpec` names the embedding (a part: tokens and positions in, residual stream
+out), the layers (each a block spec), the order in which layers run, the final
+norm, the output head and an optional step on the logits.  `DecoderModel`
 builds the parts through their registries, declares every tensor they bind,
 and runs a step's rows through the schedule.
 
@@ -18,8 +19,8 @@ from typing import Dict, List, Mapping, Optional, Sequence
 
 import torch
 
-from .parts.base import (BLOCKS, MATRIX, NORMS, Block, BuildEnv, LayerCache, Norm, PartSpec, RowStats,
-                         StepContext, TensorSpec, build_part, project)
+from .parts.base import (BLOCKS, EMBEDDINGS, LOGIT_STEPS, MATRIX, NORMS, Block, BuildEnv, Embedding, LogitsStep, Norm,
+                         PartSpec, RowStats, StepContext, TensorSpec, build_part, project)
 
 
 @dataclass(frozen=True)
@@ -32,21 +33,30 @@ class Run:
 class ModelSpec:
     vocab_size: int
     width: int
-    embedding_name: str
+    embedding: PartSpec  # an `Embedding` kind
     layers: Sequence[PartSpec]  # block specs
     schedule: Sequence[Run]
     final_norm: PartSpec
-    head_name: Optional[str]  # None: always the embedding matrix
-    tie_head: bool  # use the embedding matrix as the head (a head tensor in the file is then unexpected)
+    head_name: Optional[str]  # None: always the embedding's table
+    tie_head: bool  # use the embedding's table as the head (a head tensor in the file is then unexpected)
     stop_ids: Sequence[int] = field(default_factory=tuple)
     bos_id: Optional[int] = None
+    logits_step: Optional[PartSpec] = None  # a `LogitsStep` kind, applied to the logits after the head
+    max_positions: Optional[int] = None  # the longest sequence the architecture's configuration allows
+
+
+def token_table(name: str, vocab_size: int, width: int) -> PartSpec:
+    """The plain embedding: x = E[token]."""
+    return PartSpec("token_table", {"name": name, "vocab_size": vocab_size, "width": width})
 
 
 class DecoderModel:
     def __init__(self, spec: ModelSpec) -> None:
         self.spec = spec
+        self.embedding: Embedding = build_part(EMBEDDINGS, spec.embedding)
         self.blocks: List[Block] = [build_part(BLOCKS, b) for b in spec.layers]
         self.final_norm: Norm = build_part(NORMS, spec.final_norm)
+        self.logits_step: Optional[LogitsStep] = build_part(LOGIT_STEPS, spec.logits_step) if spec.logits_step else None
         for i, run in enumerate(spec.schedule):
             if not 0 <= run.layer < len(self.blocks):
                 raise ValueError(f"schedule names layer {run.layer}, the model has {len(self.blocks)}")
@@ -54,33 +64,43 @@ class DecoderModel:
                 if not 0 <= run.cache_of < i or spec.schedule[run.cache_of].cache_of is not None:
                     raise ValueError(f"run {i} of the schedule reads the cache of run {run.cache_of}, which is "
                                      "not an earlier run with a cache of its own")
-        self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
         self.env: Optional[BuildEnv] = None
+
+    def parts(self):
+        return (self.embedding, *self.blocks, self.final_norm, *((self.logits_step,) if self.logits_step else ()))
+
+    @property
+    def graph_safe(self) -> bool:
+        """Whether every part only launches library kernels (then decoding steps can be captured)."""
+        return all(getattr(p, "graph_safe", False) for p in self.parts())
 
     # ---- tensors ---------------------------------------------------------------
     def tensor_specs(self) -> List[TensorSpec]:
         s = self.spec
-        specs = [TensorSpec(s.embedding_name, (s.vocab_size, s.width), kind=MATRIX)]
+        specs = list(self.embedding.tensor_specs())
         for b in self.blocks:
             specs.extend(b.tensor_specs())
         specs.extend(self.final_norm.tensor_specs())
         if s.head_name is not None and not s.tie_head:
             specs.append(TensorSpec(s.head_name, (s.vocab_size, s.width), kind=MATRIX))
+        if self.logits_step is not None:
+            specs.extend(self.logits_step.tensor_specs())
         return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         self.env = env
         s = self.spec
-        self.embedding = tensors[s.embedding_name].contiguous()
-        for b in self.blocks:
-            b.bind(tensors, env)
-        self.final_norm.bind(tensors, env)
+        for p in self.parts():
+            p.bind(tensors, env)
         if s.head_name is not None and not s.tie_head:
             self.head = tensors[s.head_name].contiguous()
         else:
             # the head is the embedding when the file has none: internal/engine/engine.go:1106-1116
-            self.head = self.embedding
+            table = self.embedding.table
+            if table is None or tuple(table.shape) != (s.vocab_size, s.width):
+                raise ValueError("the output head is tied to the embedding, which has no [vocab, width] table")
+            self.head = table
 
     # ---- what the cache has to hold -----------------------------------------------
     def cache_needs(self) -> Dict[int, object]:
@@ -94,14 +114,13 @@ class DecoderModel:
         return needs
 
     # ---- one step -------------------------------------------------------------------
-    def forward(self, ctx: StepContext, caches: Mapping[int, LayerCache], want_rows: torch.Tensor,
+    def forward(self, ctx: StepContext, caches: Mapping[int, object], want_rows: torch.Tensor,
                 n_want: int) -> Optional[torch.Tensor]:
         """Runs ctx.rows tokens through the schedule; returns float32 logits [n_want, vocab]
         of the rows listed in want_rows (None when nothing is wanted)."""
         kn = ctx.kernels
         s = self.spec
-        x = ctx.ws.alloc((ctx.rows, s.width), torch.float32, keep=True)
-        kn.embed(self.embedding, ctx.tokens, x)
+        x = self.embedding.forward(ctx)
         pending: Optional[torch.Tensor] = None
         if ctx.observe is not None:
             ctx.observe("embed", x, None)
@@ -109,8 +128,7 @@ class DecoderModel:
             ctx.ws.next_run()  # the buffers of the run before the last one are free again
             cache = caches.get(i if run.cache_of is None else run.cache_of)
             if cache is not None and run.cache_of is not None:
-                cache = LayerCache(write=False, k=cache.k, v=cache.v, block_table=cache.block_table,
-                                   block_size=cache.block_size, state=cache.state)
+                cache = cache.read_only()
             block = self.blocks[run.layer]
             if block.takes_next_norm:
                 after = self.blocks[s.schedule[i + 1].layer].first_norm if i + 1 < len(s.schedule) else None
@@ -129,4 +147,6 @@ class DecoderModel:
         if logits is None:
             logits = torch.empty((n_want, s.vocab_size), dtype=torch.float32, device=ctx.device)
         project(kn, ctx, normed, self.head, logits)
+        if self.logits_step is not None:
+            self.logits_step.forward(logits, ctx)
         return logits

@@ -6,7 +6,7 @@ internal/engine/engine.go:402-433, 921-951)."""
 from __future__ import annotations
 
 from ..config.llama import LlamaConfig
-from ..model import ModelSpec, Run
+from ..model import ModelSpec, Run, token_table
 from ..parts.base import PartSpec
 from ..registry import register_architecture
 
@@ -40,7 +40,7 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
     return ModelSpec(
         vocab_size=cfg.vocab_size,
         width=cfg.hidden_size,
-        embedding_name="model.embed_tokens.weight",
+        embedding=token_table("model.embed_tokens.weight", cfg.vocab_size, cfg.hidden_size),
         layers=tuple(layers),
         schedule=tuple(Run(i) for i in range(cfg.num_hidden_layers)),
         final_norm=PartSpec("rmsnorm", {"width": cfg.hidden_size, "eps": cfg.rms_norm_eps,
@@ -49,6 +49,7 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         tie_head=cfg.tie_word_embeddings,
         stop_ids=tuple(cfg.eos_token_ids),
         bos_id=cfg.bos_token_id,
+        max_positions=cfg.max_position_embeddings,
     )
 
 

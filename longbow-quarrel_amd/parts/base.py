@@ -11,7 +11,7 @@ constructor parameters, the tensors it declared, and the `StepContext`.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass, field, replace
 from typing import Any, Callable, Dict, Generic, List, Mapping, Optional, Tuple, TypeVar
 
 import torch
@@ -56,6 +56,8 @@ FEED_FORWARDS: Registry = Registry("feed-forward")
 NORMS: Registry = Registry("norm")
 POSITION_ENCODINGS: Registry = Registry("position encoding")
 BLOCKS: Registry = Registry("block")
+EMBEDDINGS: Registry = Registry("embedding")
+LOGIT_STEPS: Registry = Registry("logits step")
 
 
 @dataclass(frozen=True)
@@ -89,8 +91,21 @@ class TensorSpec:
 # ---- what a mixer asks of the cache ----------------------------------------------
 
 
+class CacheNeed:
+    """What a mixer asks of the cache.  Needs are hashable values: runs of the schedule whose mixers
+    state equal needs share one group of storage, unequal needs get storage of their own.  A need
+    builds its own group, so a new kind of per-sequence storage is a new need class with a group
+    class beside it (`cache.CacheGroup` is the interface) and nothing else changes."""
+
+    def make_group(self, runs: List[int], n_blocks: int, max_slots: int, dtype: torch.dtype,
+                   device: torch.device):
+        """Storage for the runs of the schedule in `runs`: a pool that may hold `n_blocks` blocks of
+        `cache.BLOCK_SIZE` positions, for at most `max_slots` live sequences."""
+        raise NotImplementedError
+
+
 @dataclass(frozen=True)
-class KVNeed:
+class KVNeed(CacheNeed):
     """Keys and values per position: `kv_heads` x `head_dim` each; window = 0 keeps all positions,
     window = w keeps the last w (older blocks go back to the pool)."""
 
@@ -98,13 +113,21 @@ class KVNeed:
     head_dim: int
     window: int = 0
 
+    def make_group(self, runs, n_blocks, max_slots, dtype, device):
+        from ..cache.manager import KVGroup
+        return KVGroup(self, runs, n_blocks, max_slots, dtype, device)
+
 
 @dataclass(frozen=True)
-class StateNeed:
+class StateNeed(CacheNeed):
     """A block of fixed size per sequence, zeroed when a slot is taken."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+    def make_group(self, runs, n_blocks, max_slots, dtype, device):
+        from ..cache.manager import StateGroup
+        return StateGroup(self, runs, max_slots, device)
 
 
 # ---- build-time and step-time context ---------------------------------------------
@@ -199,6 +222,10 @@ class Workspace:
         """Bytes this step has needed so far."""
         return self.step.high + self.runs[0].high + self.runs[1].high
 
+    def fits(self) -> bool:
+        """Whether what this step has needed so far lay inside the buffers (else the next `reset` moves them)."""
+        return all(a.high <= a.buf.numel() for a in (self.step, *self.runs))
+
 
 @dataclass
 class StepContext:
@@ -225,6 +252,9 @@ class StepContext:
     max_len: int = 0
     decode: bool = False  # every sequence brings exactly one token
     logits_out: Optional[torch.Tensor] = None  # where the logits go (a captured step's fixed buffer)
+    # True while a step is only walked through to learn its workspace size: `kernels` then answers
+    # size questions and launches nothing; a part that launches kernels of its own must not either
+    dry: bool = False
     shared: Dict[Any, Any] = field(default_factory=dict)  # what parts compute once a step and share
     # debugging: called with ("embed" | "run <i>", x, pending) after the embedding and after every run of the
     # schedule; the residual stream at that point is x plus what is pending (a delta, pieces of one, or
@@ -245,6 +275,10 @@ class LayerCache:
     # fixed-size state (StateNeed)
     state: Optional[torch.Tensor] = None  # [slots, *shape]
 
+    def read_only(self) -> "LayerCache":
+        """The same storage for a run of the schedule that reads what another run wrote."""
+        return replace(self, write=False)
+
 
 # ---- the parts -----------------------------------------------------------------------
 
@@ -264,6 +298,26 @@ class Part:
         """`tensors` holds every declared name that the file had, already on the device
         and in the dtype its kind asks for."""
         self.env = env
+
+
+class Embedding(Part):
+    """forward(ctx) -> the float32 residual stream [rows, width] of the step's tokens (`ctx.tokens`, with
+    `ctx.row_pos` for an encoding that adds positions here), in a buffer from
+    `ctx.ws.alloc(..., keep=True)`.  `table` is the [vocab, width] matrix that a tied output head uses
+    (None if the embedding has none of that shape)."""
+
+    table: Optional[torch.Tensor] = None
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class LogitsStep(Part):
+    """forward(logits, ctx): changes the float32 logits [wanted, vocab] in place, after the head (a
+    scale, a soft cap)."""
+
+    def forward(self, logits: torch.Tensor, ctx: StepContext) -> None:
+        raise NotImplementedError
 
 
 class Norm(Part):

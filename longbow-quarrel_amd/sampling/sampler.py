@@ -1,7 +1,7 @@
 """Picks the next token of every sequence of a batch from its logits, on the device."""
 from __future__ import annotations
 
-from typing import Optional
+from typing import List, Optional
 
 import torch
 
@@ -9,9 +9,14 @@ from .params import SamplingParams
 from .state import SamplerState
 
 
+NO_TOKEN = -1
+
+
 class NonFiniteLogits(RuntimeError):
-    """The reference falls back to the first finite index (internal/engine/sampler.go:73-75,
-    107-123); a library that is checked for exactness reports the fault instead."""
+    """A row of logits holds a NaN or an infinity.  The reference scans for them and falls back to the
+    first finite index (internal/engine/sampler.go:73-75, 107-123); a library that is checked for
+    exactness reports the fault instead.  The kernels write `NO_TOKEN` for such a row and leave its
+    generator and its ring of recent ids alone; whoever reads the tokens back raises this."""
 
 
 class Sampler:
@@ -31,3 +36,13 @@ class Sampler:
         else:
             kn.sample(logits, out, seq_slot, p.temperature, p.top_k, p.top_p, st.rng_key, st.rng_ctr,
                       st.recent, st.recent_n)
+
+    @staticmethod
+    def read_tokens(out: torch.Tensor) -> List[int]:
+        """The sampled tokens on the host (waits for them); raises `NonFiniteLogits` naming the rows
+        whose logits could not be sampled from."""
+        tokens = out.cpu().tolist()
+        bad = [r for r, t in enumerate(tokens) if t == NO_TOKEN]
+        if bad:
+            raise NonFiniteLogits(f"the logits of row(s) {bad} hold a NaN or an infinity; nothing was sampled from them")
+        return tokens

@@ -43,10 +43,20 @@ class SafetensorsFile:
 
     def __init__(self, path: str) -> None:
         self.path = path
+        self._map = None
         size = os.path.getsize(path)
         if size < 8:
             raise WeightFileError(f"{path}: too short to be a safetensors file ({size} bytes)")
         self._f = open(path, "rb")
+        try:
+            self._read_header(size)
+            self._map = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_READ)
+        except BaseException:
+            self._f.close()  # a rejected file leaves no handle behind
+            raise
+
+    def _read_header(self, size: int) -> None:
+        path = self.path
         (hlen,) = struct.unpack("<Q", self._f.read(8))
         if hlen <= 0 or 8 + hlen > size:
             raise WeightFileError(f"{path}: header length {hlen} does not fit the file ({size} bytes)")
@@ -54,15 +64,20 @@ class SafetensorsFile:
             header = json.loads(self._f.read(hlen).decode("utf-8"))
         except (UnicodeDecodeError, json.JSONDecodeError) as e:
             raise WeightFileError(f"{path}: header is not valid JSON ({e})") from e
+        if not isinstance(header, dict):
+            raise WeightFileError(f"{path}: header is not a JSON object")
         self.metadata = header.pop("__metadata__", {})
         self.data_start = 8 + hlen
         self.entries: Dict[str, Tuple[torch.dtype, Tuple[int, ...], int, int]] = {}
         for name, info in header.items():
-            dt = info.get("dtype")
-            if dt not in _DTYPES:
-                raise WeightFileError(f"{path}: tensor {name!r} has unsupported dtype {dt!r}")
-            shape = tuple(int(s) for s in info["shape"])
-            begin, end = (int(o) for o in info["data_offsets"])
+            try:
+                dt = info.get("dtype")
+                if dt not in _DTYPES:
+                    raise WeightFileError(f"{path}: tensor {name!r} has unsupported dtype {dt!r}")
+                shape = tuple(int(s) for s in info["shape"])
+                begin, end = (int(o) for o in info["data_offsets"])
+            except (KeyError, TypeError, ValueError, AttributeError) as e:
+                raise WeightFileError(f"{path}: tensor {name!r} has a malformed header entry ({e!r})") from e
             n = 1
             for s in shape:
                 n *= s
@@ -73,7 +88,6 @@ class SafetensorsFile:
             if begin < 0 or self.data_start + end > size:
                 raise WeightFileError(f"{path}: tensor {name!r} data truncated (ends at {self.data_start + end}, file has {size})")
             self.entries[name] = (_DTYPES[dt], shape, begin, end)
-        self._map = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_READ) if size > 0 else None
 
     def names(self) -> List[str]:
         return list(self.entries)
@@ -129,7 +143,18 @@ def open_model_files(folder: str) -> List[SafetensorsFile]:
     if os.path.isfile(single):
         return [SafetensorsFile(single)]
     if os.path.isfile(index):
-        with open(index, "r", encoding="utf-8") as f:
-            shards = sorted(set(json.load(f)["weight_map"].values()))
-        return [SafetensorsFile(os.path.join(folder, s)) for s in shards]
+        try:
+            with open(index, "r", encoding="utf-8") as f:
+                shards = sorted(set(json.load(f)["weight_map"].values()))
+        except (KeyError, TypeError, AttributeError, json.JSONDecodeError) as e:
+            raise WeightFileError(f"{index}: not an index with a weight_map ({e!r})") from e
+        opened: List[SafetensorsFile] = []
+        try:
+            for s in shards:
+                opened.append(SafetensorsFile(os.path.join(folder, s)))
+        except BaseException:
+            for f in opened:  # a later shard was refused: the earlier ones are closed again
+                f.close()
+            raise
+        return opened
     raise WeightFileError(f"no model.safetensors (or model.safetensors.index.json) in {folder!r}")

@@ -12,6 +12,8 @@ from typing import Optional
 
 import torch
 
+from longbow_quarrel_amd.kernels.dry import query
+
 
 class CpuKernels:
     name = "cpu-test-standin"
@@ -31,9 +33,11 @@ class CpuKernels:
         d = delta.float()
         return d.sum(0) if d.dim() == like.dim() + 1 else d
 
+    @query
     def linear_pieces(self, dtype, m, n, k):
         return 1
 
+    @query
     def linear_fused_parts(self, dtype, m, n, k):
         return 0
 
@@ -95,6 +99,7 @@ class CpuKernels:
             kcache[blk, :, off, :] = kr[r]
             vcache[blk, :, :, off] = vr[r]
 
+    @query
     def attention_workspace(self, dtype, rows, heads, kv_heads, head_dim, block_size, decode, max_len):
         return 0
 
@@ -117,3 +122,14 @@ class CpuKernels:
                 s = (kk[:, g] @ qv) * scale
                 pr = torch.softmax(s, dim=0)
                 out[r, h * head_dim : (h + 1) * head_dim] = (pr[:, None] * vv[:, g]).sum(0).to(out.dtype)
+
+    # greedy sampling and the upkeep of a decoding batch's arrays, so that the generation loop runs here too
+    def argmax(self, logits, out, scratch=None, seq_slot=None, recent=None, recent_n=None):
+        rows = logits.shape[0]
+        best = logits.argmax(dim=-1).to(torch.int32)
+        bad = ~torch.isfinite(logits).all(dim=-1)
+        out[:rows] = torch.where(bad, torch.full_like(best, -1), best)
+
+    def advance(self, row_pos, seq_start, seq_len, batch):
+        for t in (row_pos, seq_start, seq_len):
+            t[:batch] += 1

@@ -127,8 +127,10 @@ def attention(
     v: torch.Tensor,
     window: int = 0,
     scale: Optional[float] = None,
+    rows: Optional[Sequence[int]] = None,
 ) -> torch.Tensor:
-    """Causal grouped-query attention over one whole sequence.
+    """Causal grouped-query attention over one whole sequence (`rows`: only these positions'
+    outputs are worked out, the others stay zero; for tests with thousands of keys).
 
     q[t, nh, hd], k[t, nkv, hd], v[t, nkv, hd] -> out[t, nh, hd].  Query head h
     reads kv head h // (nh / nkv); row p sees keys start..p with start = 0 or
@@ -146,7 +148,7 @@ def attention(
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
     out = torch.zeros(t, nh, hd, dtype=F64)
-    for p in range(t):
+    for p in (range(t) if rows is None else rows):
         start = p - window + 1 if (window > 0 and p >= window) else 0
         for h in range(nh):
             g = h // group

@@ -181,6 +181,86 @@ def test_truncated_and_malformed_files_are_refused(tmp_path):
         SafetensorsFile(path)
 
 
+def test_rejected_files_leave_no_open_handle_and_malformed_entries_are_weight_errors(tmp_path):
+    def open_files():
+        return len(os.listdir("/proc/self/fd"))
+
+    def write_raw(path, header):
+        blob = json.dumps(header).encode()
+        open(path, "wb").write(struct.pack("<Q", len(blob)) + blob + b"\0" * 64)
+
+    path = str(tmp_path / "m.safetensors")
+    before = open_files()
+    for header in ({"a": {"dtype": "F32", "data_offsets": [0, 4]}},  # no shape
+                   {"a": {"dtype": "F32", "shape": [1], "data_offsets": [0]}},  # one offset
+                   {"a": {"dtype": "F32", "shape": ["x"], "data_offsets": [0, 4]}},
+                   {"a": "F32"}, ["a"]):
+        write_raw(path, header)
+        with pytest.raises(WeightFileError):
+            SafetensorsFile(path)
+    assert open_files() == before
+    # a folder whose second shard is refused: the first shard is closed again
+    folder = tmp_path / "sharded"
+    folder.mkdir()
+    write_safetensors(str(folder / "a.safetensors"), {"x": torch.zeros(3)})
+    write_raw(str(folder / "b.safetensors"), {"y": {"dtype": "F32"}})
+    (folder / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"x": "a.safetensors", "y": "b.safetensors"}}))
+    from longbow_quarrel_amd.weights.safetensors_io import open_model_files
+    with pytest.raises(WeightFileError, match="b.safetensors"):
+        open_model_files(str(folder))
+    assert open_files() == before
+    (folder / "model.safetensors.index.json").write_text("{}")
+    with pytest.raises(WeightFileError, match="weight_map"):
+        open_model_files(str(folder))
+
+
+def _shard(folder, parts):
+    """Rewrites a model folder as shards with an index; `parts` maps shard file -> predicate on names."""
+    cfg, tensors = read_folder(folder)
+    os.remove(os.path.join(folder, "model.safetensors"))
+    weight_map = {}
+    for fname, take in parts.items():
+        mine = {n: t for n, t in tensors.items() if take(n)}
+        write_safetensors(os.path.join(folder, fname), mine)
+        weight_map.update({n: fname for n in mine})
+    with open(os.path.join(folder, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": weight_map}, f)
+    return tensors
+
+
+def test_a_sharded_folder_loads_to_the_same_tensors_and_a_name_in_two_shards_is_an_error(tmp_path):
+    folder = write_folder(tmp_path, TINY_B, 4)
+    model = DecoderModel(spec_from_config(config_from_dict(read_config_json(folder))))
+    whole = load_tensors(folder, model.tensor_specs(), torch.bfloat16, torch.device("cpu"))
+    first = lambda n: "layers.0." in n or "embed" in n
+    _shard(folder, {"model-00001-of-00002.safetensors": first,
+                    "model-00002-of-00002.safetensors": lambda n: not first(n)})
+    sharded = load_tensors(folder, model.tensor_specs(), torch.bfloat16, torch.device("cpu"))
+    assert sharded.keys() == whole.keys() and all(torch.equal(sharded[n], whole[n]) for n in whole)
+    # the same name in both shards
+    _, t = read_folder_shard(folder, "model-00001-of-00002.safetensors")
+    dup = "model.layers.0.mlp.up_proj.weight"
+    _, second = read_folder_shard(folder, "model-00002-of-00002.safetensors")
+    second[dup] = t[dup]
+    write_safetensors(os.path.join(folder, "model-00002-of-00002.safetensors"), second)
+    with pytest.raises(WeightError) as e:
+        load_tensors(folder, model.tensor_specs(), torch.bfloat16, torch.device("cpu"))
+    assert dup in str(e.value) and "in both" in str(e.value)
+    # a shard that lacks a tensor: the one error names it, as for a single file
+    del second[dup], second["model.norm.weight"]
+    write_safetensors(os.path.join(folder, "model-00002-of-00002.safetensors"), second)
+    with pytest.raises(WeightError) as e:
+        load_tensors(folder, model.tensor_specs(), torch.bfloat16, torch.device("cpu"))
+    assert e.value.missing == ["model.norm.weight"]
+
+
+def read_folder_shard(folder, fname):
+    sf = SafetensorsFile(os.path.join(folder, fname))
+    tensors = {n: sf.tensor(n) for n in sf.names()}
+    sf.close()
+    return None, tensors
+
+
 def test_storage_dtype_rule():
     m, v, t = TensorSpec("m", (1,)), TensorSpec("v", (1,), kind=VECTOR32), TensorSpec("t", (1,), kind=TABLE)
     bf, f32, f16 = torch.bfloat16, torch.float32, torch.float16

@@ -17,9 +17,11 @@ from longbow_quarrel_amd.weights import random_tensors
 TOL = 2e-5
 
 
-def make(tmp_path, cfg, seed=7, max_tokens=1024):
+def make(tmp_path, cfg, seed=7, max_tokens=1024, max_sequence_tokens=4096):
     folder = write_folder(tmp_path, cfg, seed, dtype=torch.float32)
-    eng = lq.load_engine(folder, dtype="float32", max_tokens=max_tokens, device="cpu", kernels=CpuKernels())
+    # the requests here are longer than the tiny configurations' max_position_embeddings: say so
+    eng = lq.load_engine(folder, dtype="float32", max_tokens=max_tokens, device="cpu", kernels=CpuKernels(),
+                         max_sequence_tokens=max_sequence_tokens)
     c, tensors = read_folder(folder)
     return eng, plain.PlainLlama(c, tensors)
 
@@ -107,14 +109,42 @@ def test_step_refuses_bad_input_and_a_full_cache_changes_nothing(tmp_path):
     assert eng.step([StepEntry(eng.new_sequence(), [3], [])]) is None  # nothing wanted, nothing returned
 
 
+def test_a_sequence_is_bounded_by_the_configuration_or_by_the_caller(tmp_path):
+    """Past `max_sequence_tokens` a step is refused before anything changes, naming the slot; the default
+    bound is the configuration's max_position_embeddings (internal/engine/kv_cache.go:121-124 refuses a
+    position past the cache's length the same way)."""
+    from longbow_quarrel_amd.engine import SequenceTooLong
+
+    eng, ref = make(tmp_path, TINY_A, max_sequence_tokens=None)
+    assert eng.max_sequence_tokens == TINY_A["max_position_embeddings"] == 128
+    toks = random_tokens(140, 256, 8)
+    a, b = eng.new_sequence(), eng.new_sequence()
+    with pytest.raises(SequenceTooLong, match=f"slot {a}"):
+        eng.step([StepEntry(a, toks[:129], [])])
+    eng.step([StepEntry(a, toks[:127], []), StepEntry(b, toks[:5], [])])
+    got = eng.step([StepEntry(a, toks[127:128], [0])])  # the 128th token still fits
+    assert rel_err(got[0], ref.forward(toks[:128])[127]) < TOL
+    with pytest.raises(SequenceTooLong, match=f"slot {a}: 128 tokens held"):
+        eng.step([StepEntry(b, [1], []), StepEntry(a, [1], [0])])
+    assert eng.length(a) == 128 and eng.length(b) == 5  # the refused step changed nothing
+    eng2, _ = make(tmp_path, TINY_A, max_sequence_tokens=10)
+    s = eng2.new_sequence()
+    with pytest.raises(SequenceTooLong):
+        eng2.step([StepEntry(s, toks[:11], [])])
+    with pytest.raises(ValueError):
+        make(tmp_path, TINY_A, max_sequence_tokens=0)
+
+
 def test_toy_parts_register_build_and_step_without_touching_the_framework(tmp_path):
     toy_parts.register_toys()
     try:
         cfg = toy_parts.ToyConfig.from_dict(toy_parts.TOY)
         eng = random_engine(cfg, seed=3, dtype="float32", max_tokens=512, device="cpu", kernels=CpuKernels(), std=0.2)
         assert not eng.graph_safe  # parts written with another library's operators are never captured
-        assert len(eng.cache.state_groups) == 1 and len(eng.cache.kv_groups) == 1
+        assert len(eng.cache.state_groups) == 1 and len(eng.cache.kv_groups) == 1 and len(eng.cache.groups) == 3
         assert sorted(eng.cache.kv_groups[0].layers) == [1, 3]  # runs 1 and 3 own keys; run 2 reads run 1's
+        latent = [g for g in eng.cache.groups if isinstance(g, toy_parts.LatentGroup)]
+        assert len(latent) == 1 and latent[0].layers == [4]  # a kind of cache the framework does not know
         tensors = random_tensors(eng.model.tensor_specs(), 3, torch.float32, 0.2)
         a, b = random_tokens(40, 53, 1), random_tokens(9, 53, 2)
         wa, wb = (toy_parts.plain_toy(toy_parts.TOY, tensors, t) for t in (a, b))
@@ -127,10 +157,123 @@ def test_toy_parts_register_build_and_step_without_touching_the_framework(tmp_pa
         out = eng.step([StepEntry(sa, a[18:], range(22))])
         assert rel_err(out, wa[18:]) < TOL
         eng.release(sa)
+        assert latent[0].blocks.taken_count == 0  # the third kind's blocks came back with the slots
         s = eng.new_sequence()  # the state of a reused slot starts from zero
         assert rel_err(eng.step([StepEntry(s, b, range(9))]), wb) < TOL
+        assert eng.max_sequence_tokens == toy_parts.TOY["positions"]
     finally:
         toy_parts.unregister_toys()
+
+
+def _replayed_graphs():
+    """Stand-ins for captured graphs on the CPU: a launch runs the step's body from the graph's own
+    arrays, as a replay does, so arrays that were not written anew give the wrong tokens here too."""
+    from longbow_quarrel_amd.engine.decode import DecodeGraph, DecodeGraphs
+
+    log = []
+
+    class ReplayedGraph(DecodeGraph):
+        def load(self, slots, tokens, starts):
+            log.append(("load", self.batch, tuple(slots)))
+            super().load(slots, tokens, starts)
+
+        def capture(self, sampler):
+            log.append(("capture", self.batch))
+            self._sampler = sampler
+            self.handle = 1
+
+        def launch(self):
+            log.append(("launch", self.batch))
+            self.run_body(self._sampler)
+
+        def destroy(self):
+            self.handle = None
+
+    class ReplayedGraphs(DecodeGraphs):
+        graph_cls = ReplayedGraph
+
+    return ReplayedGraphs, log
+
+
+@pytest.mark.parametrize("n_prompts,max_batch", [(6, 3), (2, 1), (5, 2)])
+def test_a_batch_after_another_of_the_same_size_loads_its_graph_anew(tmp_path, n_prompts, max_batch):
+    """Several batches of one size in one call: the second finds a graph of its size, on the same slots,
+    whose arrays still hold the first batch's last tokens and positions.  Its first decoding step must
+    write them anew.  Greedy tokens with graphs equal those of direct steps and of the plain model."""
+    from longbow_quarrel_amd.engine.generate import EngineBackend, GenerationLoop
+
+    eng, ref = make(tmp_path, TINY_A)
+    assert eng.graph_safe
+    prompts = [random_tokens(3 + 2 * i, 256, 40 + i) for i in range(n_prompts)]
+    expect = []
+    for p in prompts:
+        seq, out = list(p), []
+        for _ in range(4):
+            out.append(plain.arg_max(ref.forward(seq)[-1]))
+            seq.append(out[-1])
+        expect.append(out)
+    graphs_cls, log = _replayed_graphs()
+    for use_graphs in (False, True):
+        be = EngineBackend(eng, lq.SamplingParams(), use_graphs=use_graphs, graphs_cls=graphs_cls)
+        assert be.use_graphs == use_graphs
+        res = GenerationLoop(be, max_batch=max_batch).run(prompts, 4, stop_ids=[])
+        be.close()
+        assert res.tokens == expect, use_graphs
+    batches = -(-n_prompts // max_batch)
+    loads = [e for e in log if e[0] == "load"]
+    assert len(loads) == batches  # once a batch: no sequence ended early, so nothing else asks for one
+    assert eng.cache.slots.taken_count == 0
+
+
+def test_prompts_run_in_portions_of_at_most_max_prefill_rows(tmp_path):
+    """A batch's prompts are fed in steps of a bounded number of rows: several sequences a step, a long
+    prompt over several steps (cut at 2 tokens, at a cache block's edge, anywhere), logits only from each
+    prompt's last portion.  The tokens do not depend on the cutting."""
+    eng, ref = make(tmp_path, TINY_C)
+    prompts = [random_tokens(n, 331, 60 + n) for n in (150, 3, 64, 1, 70)]
+    whole = lq.generate(eng, prompts, 3, stop_ids=[], use_graphs=False)
+    expect = []
+    for p in prompts:
+        seq, out = list(p), []
+        for _ in range(3):
+            out.append(plain.arg_max(ref.forward(seq)[-1]))
+            seq.append(out[-1])
+        expect.append(out)
+    assert whole.tokens == expect
+    from longbow_quarrel_amd.engine.generate import EngineBackend, GenerationLoop
+    for rows, steps in ((2, 144), (64, 5), (100, 3), (1000, 1)):  # the 288 rows, densely packed
+        be = EngineBackend(eng, lq.SamplingParams(), use_graphs=False, max_prefill_rows=rows)
+        res = GenerationLoop(be).run(prompts, 3, stop_ids=[])
+        assert res.tokens == expect, rows
+        assert be.prefill_steps == steps, (rows, be.prefill_steps)
+    with pytest.raises(ValueError):
+        EngineBackend(eng, lq.SamplingParams(), max_prefill_rows=0)
+
+
+def test_generation_stops_where_a_sequence_may_not_grow_further(tmp_path):
+    from longbow_quarrel_amd.engine import SequenceTooLong
+
+    eng, ref = make(tmp_path, TINY_A, max_sequence_tokens=12)
+    a, b = random_tokens(10, 256, 1), random_tokens(4, 256, 2)
+    res = lq.generate(eng, [a, b], 6, stop_ids=[], use_graphs=False)
+    # 10 prompt tokens + 2 fed back fill the 12; the third token is sampled and never fed
+    assert [len(t) for t in res.tokens] == [3, 6] and res.finish == ["length", "length"]
+    with pytest.raises(SequenceTooLong, match="request 1"):
+        lq.generate(eng, [b, a + a], 2, stop_ids=[], use_graphs=False)
+    assert eng.cache.slots.taken_count == 0
+
+
+def test_non_finite_logits_are_reported_not_sampled(tmp_path):
+    """A NaN or an infinity among a row's logits stops generation with an error that names the request
+    (the reference would go on from the first finite index: internal/engine/sampler.go:72-75, 107-123)."""
+    folder = write_folder(tmp_path, TINY_A, 5, dtype=torch.float32)
+    c, tensors = read_folder(folder)
+    eng = lq.load_engine(folder, dtype="float32", max_tokens=512, device="cpu", kernels=CpuKernels())
+    assert lq.generate(eng, [[1, 2, 3], [4, 5]], 3, stop_ids=[], use_graphs=False).finish == ["length"] * 2
+    eng.model.head[17, :] = float("inf")  # token 17's logit overflows for every row
+    with pytest.raises(lq.NonFiniteLogits, match="request 0"):
+        lq.generate(eng, [[1, 2, 3], [4, 5]], 3, stop_ids=[], use_graphs=False)
+    assert eng.cache.slots.taken_count == 0  # the failed call gave its slots back
 
 
 def test_workspace_lifetimes():

@@ -260,7 +260,7 @@ def paged_cache(lengths, kv_heads, head_dim, dtype, seed):
 
 
 def run_attention(kn, q_rows, lengths, new, heads, kv_heads, head_dim, dtype, seed, window=0, decode=False,
-                  force_generic=False, standout=None):
+                  force_generic=False, standout=None, max_len=None):
     """q rows for the last `new[b]` positions of each sequence; returns (got, want)."""
     kc, vc, table, slots, dense = paged_cache(lengths, kv_heads, head_dim, dtype, seed)
     g = torch.Generator().manual_seed(seed + 1)
@@ -286,11 +286,12 @@ def run_attention(kn, q_rows, lengths, new, heads, kv_heads, head_dim, dtype, se
     out = torch.empty_like(qd)
     scale = 1.0 / math.sqrt(head_dim)
     kn.force_generic = force_generic
+    max_len = max_len or max(lengths)
     try:
-        need = kn.attention_workspace(dtype, rows, heads, kv_heads, head_dim, BS, decode, max(lengths))
+        need = kn.attention_workspace(dtype, rows, heads, kv_heads, head_dim, BS, decode, max_len)
         ws = torch.empty(need, dtype=torch.float32, device=DEV) if need else None
         kn.attention(qd, out, heads, kv_heads, head_dim, i32(row_pos), i32(row_seq), i32(slots), i32(cu),
-                     table, kc, vc, BS, scale, window, decode=decode, max_len=max(lengths), workspace=ws)
+                     table, kc, vc, BS, scale, window, decode=decode, max_len=max_len, workspace=ws)
     finally:
         kn.force_generic = False
     want = torch.zeros((rows, heads, head_dim), dtype=torch.float64)
@@ -300,7 +301,7 @@ def run_attention(kn, q_rows, lengths, new, heads, kv_heads, head_dim, dtype, se
         # plain attention over the whole sequence with the real queries in the last m places
         qfull = torch.zeros((n, heads, head_dim), dtype=torch.float64)
         qfull[n - m:] = q[r : r + m].double().view(m, heads, head_dim)
-        want[r : r + m] = plain.attention(qfull, k, v, window=window)[n - m:]
+        want[r : r + m] = plain.attention(qfull, k, v, window=window, rows=range(n - m, n))[n - m:]
         r += m
     return out.view(rows, heads, head_dim), want
 
@@ -345,6 +346,26 @@ def test_decode_attention_over_several_splits(kn, head_dim, heads, kv_heads, win
                              window=window, decode=True)
     assert torch.equal(got, again)
     assert int(kn._tickets.abs().max()) == 0
+
+
+@pytest.mark.parametrize("rows", [24, 64])
+def test_decode_attention_of_many_rows_with_long_splits(kn, rows):
+    """24 and 64 sequences of 8 kv heads and head size 128, up to 3 000 keys: so many workgroups that a
+    split covers 512 to 3 072 positions (one split for some launches, several for others, with rows of one
+    launch ending in different splits).  Twice, with the ticket counters back at zero after each."""
+    g = torch.Generator().manual_seed(rows)
+    lengths = torch.randint(1, 3001, (rows,), generator=g).tolist()
+    lengths[0], lengths[1], lengths[2] = 3000, 1, 1025
+    for max_extra in (0, 1100):  # the bound a captured step would pass: lengths rounded up, or a bucket more
+        got, want = run_attention(kn, None, lengths, [1] * rows, 32, 8, 128, torch.bfloat16, 61, decode=True,
+                                  max_len=max(lengths) + max_extra)
+        assert rel_err(got, want) < 8e-3
+        for r in (0, 1, 2, rows - 1):  # row by row: a row that a split lost would drown in the whole
+            assert rel_err(got[r], want[r]) < 8e-3, (r, lengths[r])
+        assert int(kn._tickets.abs().max()) == 0
+    again, _ = run_attention(kn, None, lengths, [1] * rows, 32, 8, 128, torch.bfloat16, 61, decode=True,
+                             max_len=max(lengths) + 1100)
+    assert torch.equal(got, again)
 
 
 @pytest.mark.parametrize("dtype,generic", [(torch.float32, True), (torch.bfloat16, False)])

@@ -162,6 +162,29 @@ def test_llama3_scaling_invariants():
     assert all(a >= b for a, b in zip(sc.tolist(), sc.tolist()[1:]))  # still non-increasing
 
 
+def test_llama3_blend_at_hand_worked_points():
+    """Inside the blend the weight is linear in original / wavelength (not in the wavelength): with low 1,
+    high 4 and factor 8, original / wavelength = 2.5 gives s = (2.5 - 1) / (4 - 1) = 0.5 and
+    f' = 0.5 f / 8 + 0.5 f = 0.5625 f; 1.75 gives s = 0.25 and f' = 0.75 f / 8 + 0.25 f = 0.34375 f.
+    (A blend linear in the wavelength would give 0.825 f and 0.5 f.)  Both the plain function and the
+    engine's table are held to these."""
+    from longbow_quarrel_amd.parts.rope import rotary_frequencies
+
+    hd, theta = 32, 500000.0
+    base = plain.rope_frequencies(hd, theta)
+    for ratio, want in ((2.5, 0.5625), (1.75, 0.34375), (1.0, 0.125), (4.0, 1.0)):
+        for i in (3, 7, 12):
+            f = float(base[i])
+            original = ratio * 2 * math.pi / f  # so that original / wavelength_i is the ratio
+            got = float(plain.llama3_scaled_frequencies(base, 8.0, 1.0, 4.0, original)[i])
+            assert math.isclose(got / f, want, rel_tol=1e-12), (ratio, i)
+            table = rotary_frequencies(hd, theta, {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                                   "high_freq_factor": 4.0,
+                                                   "original_max_position_embeddings": original})
+            assert math.isclose(table[i] / f, want, rel_tol=1e-12), (ratio, i)
+            assert math.isclose(table[0], 1.0) and len(table) == hd // 2
+
+
 def test_llama3_scaling_reduces_to_identity():
     base = plain.rope_frequencies(64, 10000.0)
     assert torch.allclose(plain.llama3_scaled_frequencies(base, 1.0, 1.0, 4.0, 64), base, rtol=1e-15)

@@ -172,3 +172,43 @@ def test_penalty_ring_holds_the_last_64_ids(kn):
     assert torch.equal(lg[0], want) and float(lg[0, 150]) == -4.0 and float(lg[0, 37]) == 1.0 and float(lg[0, 38]) == 0.5
     # the sampled token joins the ring
     assert int(state.recent_n[0]) == 103 and tok[0] in state.recent[0].cpu().tolist()
+
+
+# --------------------------------------------------------------------------- rows that cannot be sampled from
+
+@pytest.mark.parametrize("params", [SamplingParams(), SamplingParams(temperature=0.8, seed=3),
+                                    SamplingParams(temperature=0.7, top_k=40, top_p=0.95, repetition_penalty=1.1, seed=3)])
+@pytest.mark.parametrize("vocab", [331, 128256])
+def test_a_row_with_a_nan_or_an_infinity_gives_no_token_and_leaves_its_state_alone(kn, params, vocab):
+    """The reference scans the logits for NaN and infinities before anything else
+    (internal/engine/sampler.go:72-75, 107-123) and then falls back; here such a row yields NO_TOKEN, its
+    generator and its ring stay as they were, and the clean rows beside it come out as if it were not there."""
+    from longbow_quarrel_amd.sampling import NonFiniteLogits
+
+    g = torch.Generator().manual_seed(vocab)
+    clean = torch.randn((5, vocab), generator=g) * 3
+    history = [[1, 2, 3]] * 5
+
+    def sample(logits):
+        state = SamplerState(5, DEV)
+        for s in range(5):
+            state.start(s, sequence_key(params.seed, s), history[s])
+        sampler = Sampler(kn, state, params)
+        out = torch.full((5,), -7, dtype=torch.int32, device=DEV)
+        sampler.sample(logits.clone().to(DEV), torch.arange(5, dtype=torch.int32, device=DEV), out)
+        return sampler, out, state
+
+    _, want, clean_state = sample(clean)
+    assert Sampler.read_tokens(want) == want.tolist() and min(want.tolist()) >= 0
+    bad = clean.clone()
+    bad[1, vocab - 1] = float("nan")  # the very last entry, the row's unaligned tail
+    bad[3, 5] = float("inf")
+    bad[4, 0] = float("-inf")
+    sampler, out, state = sample(bad)
+    assert out.tolist() == [want[0].item(), -1, want[2].item(), -1, -1]
+    with pytest.raises(NonFiniteLogits, match=r"row\(s\) \[1, 3, 4\]"):
+        Sampler.read_tokens(out)
+    # the rows that were refused: no draw taken, nothing pushed into the ring
+    assert state.rng_ctr.tolist()[1] == 0 and state.recent_n.tolist()[1] == 3
+    assert state.rng_ctr.tolist()[0] == clean_state.rng_ctr.tolist()[0]
+    assert state.recent_n.tolist()[0] == 4 and state.recent_n.tolist()[3] == 3
