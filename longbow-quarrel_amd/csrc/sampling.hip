@@ -21,6 +21,9 @@
 // the random numbers (counter-based: draw n of a sequence depends on key and n only) and a ring
 // of the last 64 token ids.
 #include "common.h"
+#include "lq_no_alloc.h"
+
+#include <mutex>
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -764,6 +767,49 @@ extern "C" int lq_argmax(const float* logits, int ld, int rows, int V, const int
   argmax_part_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, stream>>>(logits, ld, V, scratch);
   argmax_final_kernel<<<rows, 64, 0, stream>>>(scratch, seq_slot, out, recent, recent_n);
   LQ_CHECK_LAUNCH("argmax");
+  return 0;
+}
+
+// ---- arg-max for callers that cannot allocate (lq_no_alloc.h) ----
+// The stages' scratch: a fixed array in device memory, a copy on every GPU, each at its own address.
+// `scratch` itself is a host-side stand-in and no device address: the pointer that kernels and other
+// HIP calls take comes from hipGetSymbolAddress, asked once per device and kept.
+static __device__ __align__(256) unsigned long long scratch[LQ_ARGMAX_NO_ALLOC_MAX_ROWS * ARGMAX_PARTS];
+
+constexpr int MAX_DEVICES = 64;
+static unsigned long long* scratch_on_device[MAX_DEVICES];  // null until the first call on that device
+static std::mutex scratch_lock;
+
+// the current device's copy of `scratch`
+static int scratch_pointer(unsigned long long** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  LQ_REQUIRE(e == hipSuccess, "argmax_no_alloc: no current device: %s", hipGetErrorString(e));
+  LQ_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "argmax_no_alloc: device %d is beyond the %d this library keeps scratch for",
+             dev, MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (scratch_on_device[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    LQ_REQUIRE(e == hipSuccess && p != nullptr, "argmax_no_alloc: the scratch array has no address on device %d: %s", dev,
+               hipGetErrorString(e));
+    scratch_on_device[dev] = (unsigned long long*)p;
+  }
+  *ptr = scratch_on_device[dev];
+  return 0;
+}
+
+extern "C" int lq_argmax_no_alloc(const float* logits, int ld, int rows, int V, int* out, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && V > 0 && ld >= V, "argmax_no_alloc: bad sizes");
+  LQ_REQUIRE(rows <= LQ_ARGMAX_NO_ALLOC_MAX_ROWS,
+             "argmax_no_alloc: %d rows are more than the %d that the fixed scratch array holds (use lq_argmax with a "
+             "scratch buffer of your own)", rows, LQ_ARGMAX_NO_ALLOC_MAX_ROWS);
+  LQ_REQUIRE(logits != nullptr && out != nullptr, "argmax_no_alloc: null pointer");
+  unsigned long long* part = nullptr;
+  if (scratch_pointer(&part) != 0) return -1;
+  argmax_part_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, stream>>>(logits, ld, V, part);
+  argmax_final_kernel<<<rows, 64, 0, stream>>>(part, nullptr, out, nullptr, nullptr);
+  LQ_CHECK_LAUNCH("argmax_no_alloc");
   return 0;
 }
 
