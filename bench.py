@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the Llama 3 8B shape on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape 8b|1b|70b]
 
 Default run: the 8B layer sizes with random bfloat16 weights, a batch of 8
 sequences that start from 512-token random prompts; W untimed decode steps, then
@@ -9,6 +9,12 @@ greedy sampling on the device and state upkeep, replayed as a HIP graph, tokens 
 back by the host every step as generation does).  `value` is decoded tokens a
 second.  The same line carries a 2,048-token prefill, the decode step's HBM
 roofline, and decode at batch 1 and 64.  One JSON line on stdout.
+
+`--shape 1b`: the Llama 3.2 1B layer sizes, 16 prompts of 64 to 4,096 tokens (uniform, from a
+seed) and then K decoding steps, all of it through the generation loop (`GenerationLoop.run`:
+prompts in portions of 8,192 rows, captured decoding steps); once with W steps untimed, then timed.
+`--shape 70b`: the 70B layer sizes, batch 8 from 1,024-token prompts, with batch 1 and a
+2,048-token prefill as points.
 """
 from __future__ import annotations
 
@@ -70,10 +76,12 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the 8B shape has (0 = all 32)")
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--batch", type=int, default=0, help="sequences a decoding step (default: 8; 16 for --shape 1b)")
+    ap.add_argument("--prompt-len", type=int, default=0,
+                    help="prompt tokens (default: 512; 1024 for --shape 70b; the shortest, 64, for --shape 1b)")
     ap.add_argument("--prompt-len-max", type=int, default=0,
-                    help="prompts of unequal lengths, uniform in [--prompt-len, this] (0 = all of --prompt-len)")
+                    help="prompts of unequal lengths, uniform in [--prompt-len, this] (0 = all of --prompt-len; "
+                         "4096 for --shape 1b)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (the headline run is 8b)")
     ap.add_argument("--no-points", action="store_true", help="skip the prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true", help="run the prefill alone, twice (for profiling)")
@@ -83,11 +91,16 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    through_loop = args.shape == "1b"  # the workload with unequal prompts runs through the generation loop
+    args.batch = args.batch or (16 if args.shape == "1b" else 8)
+    args.prompt_len = args.prompt_len or {"8b": 512, "1b": 64, "70b": 1024}[args.shape]
+    if args.shape == "1b" and not args.prompt_len_max:
+        args.prompt_len_max = 4096
 
     import torch
 
     import longbow_quarrel_amd as lq
-    from longbow_quarrel_amd.engine import EngineBackend, StepEntry
+    from longbow_quarrel_amd.engine import EngineBackend, GenerationLoop, StepEntry
 
     cfg = dict(SHAPES[args.shape])
     full_layers = cfg["num_hidden_layers"]
@@ -95,7 +108,7 @@ def main() -> int:
         cfg["num_hidden_layers"] = args.layers
     config = lq.LlamaConfig.from_dict(cfg)
     slot_len = cfg["max_position_embeddings"]
-    max_batch = 64 if not (args.no_points or args.prefill_only) else args.batch
+    max_batch = 64 if (args.shape == "8b" and not (args.no_points or args.prefill_only)) else args.batch
     t0 = time.time()
     engine = lq.random_engine(config, seed=0, dtype="bfloat16", max_tokens=max_batch * slot_len, max_slots=max_batch)
     torch.cuda.synchronize()
@@ -113,11 +126,7 @@ def main() -> int:
         if args.prompt_len_max > prompt_len:
             lens = torch.randint(prompt_len, args.prompt_len_max + 1, (batch,), generator=gen).tolist()
         prompts = [random_prompt(n) for n in lens]
-        # prompts in chunks of sequences so that a prefill step stays at a few thousand rows
-        toks = []
-        per = max(1, 4096 // max(lens))
-        for i in range(0, batch, per):
-            toks += backend.prefill(slots[i : i + per], prompts[i : i + per])
+        toks = backend.prefill(slots, prompts)  # in portions of at most 8,192 rows a step
         for _ in range(warmup):
             toks = backend.decode(slots, toks, False)
         torch.cuda.synchronize()
@@ -144,15 +153,7 @@ def main() -> int:
         torch.cuda.synchronize()
         print(f"[bench] prefill of {n} tokens: {(time.perf_counter() - t) * 1e3:.2f} ms", file=sys.stderr, flush=True)
         return 0
-    value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
-    step_bytes = weight_bytes_per_step(config) + args.batch * ctx_mean * kv_bytes_per_token(config)
-    achieved = step_bytes / (ms_step * 1e-3) / 1e9
-    print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
-
-    prefill = None
-    points = {}
-    if not args.no_points:
-        t_tokens = 2048
+    def prefill_point(t_tokens: int):
         slot = engine.new_sequence()
         prompt = random_prompt(t_tokens)
         # once untimed (first launches), then three times on fresh slots: the median
@@ -168,18 +169,51 @@ def main() -> int:
             times.append(time.perf_counter() - t)
             engine.release(slot)
         dt = sorted(times)[1]
-        prefill = {
-            "value": round(t_tokens / dt, 1), "tokens": t_tokens, "ms": round(dt * 1e3, 3),
-            "frac": round(prefill_flops(config, t_tokens) / dt / (BF16_TFLOPS * 1e12), 4),
-        }
+        return {"value": round(t_tokens / dt, 1), "tokens": t_tokens, "ms": round(dt * 1e3, 3),
+                "frac": round(prefill_flops(config, t_tokens) / dt / (BF16_TFLOPS * 1e12), 4)}
+
+    prefill = None
+    points = {}
+    if through_loop:
+        # 16 prompts of unequal lengths, then decoding, as one call of the generation loop; the untimed
+        # call before it leaves the captured steps behind for the timed one
+        lens = torch.randint(args.prompt_len, args.prompt_len_max + 1, (args.batch,), generator=gen).tolist()
+        prompts = [random_prompt(n) for n in lens]
+        backend = EngineBackend(engine, lq.SamplingParams(temperature=0.0), use_graphs=True)
+        loop = GenerationLoop(backend, max_batch=args.batch)
+        loop.run(prompts, args.warmup + 1, stop_ids=[])
+        torch.cuda.synchronize()
+        res = loop.run(prompts, args.steps + 1, stop_ids=[])  # the first token comes from the prompts' step
+        backend.close()
+        assert res.decode_steps == args.steps and res.batches == 1
+        ms_step = res.decode_seconds / res.decode_steps * 1e3
+        value = args.batch * res.decode_steps / res.decode_seconds
+        ctx_mean = sum(lens) / args.batch + (args.steps + 1) / 2.0
+        n_prompt = res.prefill_tokens
+        flops = sum(prefill_flops(config, n) for n in lens)
+        prefill = {"value": round(n_prompt / res.prefill_seconds, 1), "tokens": n_prompt,
+                   "ms": round(res.prefill_seconds * 1e3, 3),
+                   "frac": round(flops / res.prefill_seconds / (BF16_TFLOPS * 1e12), 4)}
+    else:
+        value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
+    step_bytes = weight_bytes_per_step(config) + args.batch * ctx_mean * kv_bytes_per_token(config)
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
+
+    if not args.no_points and not through_loop:
+        prefill = prefill_point(2048)
         print(f"[bench] prefill: {prefill}", file=sys.stderr, flush=True)
         v1, _, _ = decode_run(1, args.prompt_len, max(16, args.steps // 2), max(4, args.warmup // 2))
-        v64, _, _ = decode_run(64, args.prompt_len, max(16, args.steps // 4), max(4, args.warmup // 2))
-        points = {"decode_b1": round(v1, 1), "decode_b64": round(v64, 1)}
+        points = {"decode_b1": round(v1, 1)}
+        if args.shape == "8b":
+            v64, _, _ = decode_run(64, args.prompt_len, max(16, args.steps // 4), max(4, args.warmup // 2))
+            points["decode_b64"] = round(v64, 1)
         print(f"[bench] points: {points}", file=sys.stderr, flush=True)
 
     line = {
-        "metric": f"decode tok/s (Llama-3 {args.shape.upper()} shape, bf16, batch {args.batch}, {args.prompt_len}-token prompts)",
+        "metric": f"decode tok/s (Llama-3 {args.shape.upper()} shape, bf16, batch {args.batch}, " + (
+            f"prompts of {args.prompt_len} to {args.prompt_len_max} tokens)" if args.prompt_len_max > args.prompt_len
+            else f"{args.prompt_len}-token prompts)"),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic: random weights N(0, 0.02) from a seed, uniform random token ids",
@@ -189,7 +223,9 @@ def main() -> int:
             "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
             "intermediate": config.intermediate_size, "vocab": config.vocab_size,
             "rope_theta": config.rope_theta, "rms_eps": config.rms_norm_eps, "tied": config.tie_word_embeddings,
-            "global_batch": args.batch, "seq_len": args.prompt_len, "context": slot_len,
+            "rope_scaling": f"{config.rope_scaling.rope_type} x{config.rope_scaling.factor:g}" if config.rope_scaling else "none",
+            "global_batch": args.batch, "seq_len": args.prompt_len,
+            "seq_len_max": max(args.prompt_len, args.prompt_len_max), "context": slot_len,
             "new_tokens": args.steps + args.warmup, "sampling": "greedy", "parallelism": "single-gpu",
         },
         "prefill": prefill,

@@ -84,7 +84,7 @@ class DecodeGraph:
         e = self.engine
         ctx = self.context()
         self.ws.reset()
-        e.model.forward(ctx, e.cache.layer_views(), self.views[7], self.batch)
+        e.forward(ctx, self.views[7], self.batch)
         sampler.sample(self.logits, self.views[3], self.views[0])
         e.kernels.advance(self.views[2], self.views[4], self.views[5], self.batch)
 
@@ -93,7 +93,7 @@ class DecodeGraph:
         what does not fit comes from the allocator for the walk); False if the workspace was too small."""
         e = self.engine
         self.ws.reset()
-        e.model.forward(self.context(dry=True), e.cache.layer_views(), self.views[7], self.batch)
+        e.forward(self.context(dry=True), self.views[7], self.batch)
         return self.ws.fits()
 
     def capture(self, sampler: Sampler) -> None:

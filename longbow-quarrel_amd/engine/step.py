@@ -177,6 +177,10 @@ class Engine:
             host_new=list(new), max_new=max(new), max_len=max_len, decode=all(n == 1 for n in new),
             logits_out=logits_out, observe=observe, dry=dry)
 
+    def forward(self, ctx: StepContext, want_rows: torch.Tensor, n_want: int) -> Optional[torch.Tensor]:
+        """The model over one step's rows, from this engine's cache."""
+        return self.model.forward(ctx, self.cache.layer_views(), want_rows, n_want)
+
     def _step(self, entries: Sequence[StepEntry], observe=None) -> Optional[torch.Tensor]:
         cache = self.cache
         growth = {e.slot: len(e.tokens) for e in entries}
@@ -205,7 +209,7 @@ class Engine:
         self.ws.reset()
         ctx = self.make_context(self.ws, (d_tokens, d_row_seq, d_row_pos, d_slot, d_start, d_len, d_cu), slots,
                                 starts, [len(e.tokens) for e in entries], max(lens), observe=observe)
-        logits = self.model.forward(ctx, cache.layer_views(), d_want, len(want_rows))
+        logits = self.forward(ctx, d_want, len(want_rows))
         cache.advance(growth)
         self.steps_run += 1
         return logits

@@ -496,3 +496,4 @@ def test_decode_attention_with_rotation_and_cache_write_folded_in(kn, heads, kv_
                  BS, scale, window, decode=True, max_len=max(lengths), workspace=ws, k_new=k2, v_new=v2, cos_sin=cs)
     assert torch.equal(kc, kc2) and torch.equal(vc, vc2)  # the same rows of the cache were written, with the same bits
     assert rel_err(out_b, out_a.double().cpu()) < 4e-3
+
