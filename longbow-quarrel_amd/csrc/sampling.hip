@@ -392,6 +392,116 @@ __device__ inline unsigned long long find_theta(const P& pass, unsigned long lon
   return theta;
 }
 
+// The threshold and the draw on a short list of (logit, index), ascending by index, by one wave.  The
+// list must hold the kept set, and whatever it holds besides must rank below it (then the longest allowed
+// prefix of the list's descending order is that of the row's).
+struct ListResult {
+  int tok, kept;
+  double mass;
+};
+
+__device__ inline ListResult list_draw(const float* list_val, const int* list_idx, int n_list, unsigned long long theta,
+                                       float mx, float invT, double u);
+
+__device__ inline ListResult list_threshold_and_draw(const float* list_val, const int* list_idx, int n_list,
+                                                     unsigned long long best, float mx, float invT, long long k_limit,
+                                                     double e_floor, bool use_p, double p_mass, double u) {
+  const int lane = threadIdx.x & 63;
+  ListPass pass{list_val, list_idx, n_list, mx, invT};
+  unsigned long long lo_key = ~0ull;
+  for (int j = lane; j < n_list; j += 64) {
+    const unsigned long long k = key_of(list_val[j], list_idx[j]);
+    lo_key = k < lo_key ? k : lo_key;
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned long long o = shfl_xor_u64(lo_key, off);
+    lo_key = o < lo_key ? o : lo_key;
+  }
+  const unsigned long long theta = find_theta(pass, best, lo_key >> 32, k_limit, e_floor, use_p, p_mass);
+  return list_draw(list_val, list_idx, n_list, theta, mx, invT, u);
+}
+
+// The same threshold for a list of a few dozen entries, without a search: every entry's rank and the mass
+// of the entries before it in the descending order, by comparing it with all others (reads of one LDS
+// word by all lanes at a time).  An entry is kept if fewer than k_limit rank before it, it is above the
+// floor, and the mass before it is below the top_p mass: the longest allowed prefix, entry by entry.
+__device__ inline unsigned long long list_threshold_by_ranks(const float* list_val, const int* list_idx, int n_list,
+                                                             float mx, float invT, long long k_limit, double e_floor,
+                                                             bool use_p, double p_mass, unsigned long long* key_sh,
+                                                             float* e_sh) {
+  const int lane = threadIdx.x & 63;
+  // every entry's key and weight once (key_sh, e_sh: n_list entries of LDS that this wave owns)
+  for (int j = lane; j < n_list; j += 64) {
+    key_sh[j] = key_of(list_val[j], list_idx[j]);
+    e_sh[j] = expf((list_val[j] - mx) * invT);
+  }
+  unsigned long long theta = ~0ull;  // the smallest kept key
+  for (int i0 = 0; i0 < n_list; i0 += 64) {
+    const int i = i0 + lane;
+    const bool has = i < n_list;
+    const unsigned long long ki = has ? key_sh[i] : ~0ull;
+    int rank = 0;
+    double before = 0.0;
+    for (int j = 0; j < n_list; ++j) {
+      const bool ahead = key_sh[j] > ki;
+      rank += ahead ? 1 : 0;
+      before += ahead ? (double)e_sh[j] : 0.0;  // in index order
+    }
+    const bool kept = has && rank < k_limit && (double)e_sh[min(i, n_list - 1)] > e_floor && (!use_p || before < p_mass);
+    if (kept && ki < theta) theta = ki;
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned long long o = shfl_xor_u64(theta, off);
+    theta = o < theta ? o : theta;
+  }
+  return theta;  // ~0: nothing is kept (then the draw falls back to the maximum)
+}
+
+__device__ inline ListResult list_draw(const float* list_val, const int* list_idx, int n_list, unsigned long long theta,
+                                       float mx, float invT, double u) {
+  const int lane = threadIdx.x & 63;
+  // the draw: running sum over the kept entries in index order, a contiguous run of the list a lane
+  const int chunk = (n_list + 63) / 64;
+  const int j0 = min(n_list, lane * chunk), j1 = min(n_list, j0 + chunk);
+  double mine = 0.0;
+  int cnt = 0;
+  for (int j = j0; j < j1; ++j)
+    if (key_of(list_val[j], list_idx[j]) >= theta) {
+      mine += (double)expf((list_val[j] - mx) * invT);
+      ++cnt;
+    }
+  double incl = mine;
+  for (int off = 1; off < 64; off <<= 1) {
+    const unsigned long long bits = (unsigned long long)__double_as_longlong(incl);
+    const unsigned hi32 = __shfl_up((unsigned)(bits >> 32), off, 64);
+    const unsigned lo32 = __shfl_up((unsigned)bits, off, 64);
+    const double o = __longlong_as_double((long long)(((unsigned long long)hi32 << 32) | lo32));
+    if (lane >= off) incl += o;
+  }
+  const double all = shfl_f64(incl, 63);  // the mass of the kept set
+  int kept = cnt;
+  for (int off = 32; off > 0; off >>= 1) kept += __shfl_xor(kept, off, 64);
+  const double r = u * all;
+  const double lo_excl = incl - mine;
+  int tok = -1;
+  if (cnt > 0 && r >= lo_excl && r < incl) {
+    double acc = lo_excl;
+    for (int j = j0; j < j1; ++j)
+      if (key_of(list_val[j], list_idx[j]) >= theta) {
+        acc += (double)expf((list_val[j] - mx) * invT);
+        tok = list_idx[j];
+        if (r < acc) break;
+      }
+  }
+  // at most one lane's range holds r
+  for (int off = 32; off > 0; off >>= 1) tok = max(tok, __shfl_xor(tok, off, 64));
+  ListResult res;
+  res.tok = tok;
+  res.kept = kept;
+  res.mass = all;
+  return res;
+}
+
 // Histogram of the row over (max - logit): bin width chosen so that every candidate (p > 1e-10) falls
 // into the bins before the last.  Counts and masses are integers (mass in units of 2^-40), so that the
 // order of the atomic additions does not matter.
@@ -399,7 +509,7 @@ constexpr int HIST_BINS = 1024;
 constexpr int LIST_CAP = 6144;   // entries of the short list in LDS
 constexpr double MASS_UNIT = 1099511627776.0;  // 2^40
 
-__global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a) {
+__global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a, const int* only) {
   __shared__ unsigned long long smu[THREADS / 64];
   __shared__ double smd[THREADS / 64];
   __shared__ double scan[THREADS];
@@ -414,6 +524,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a) {
   __shared__ int tok_sh, kept_sh;
   __shared__ double total_sh;
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (only != nullptr && only[row] == 0) return;  // the parts have dealt with this row
   const float* lr = a.logits + (long long)row * a.ld;
   const int V = a.V;
   const float invT = a.inv_temperature;
@@ -606,56 +717,12 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a) {
     __syncthreads();
     // one wave finds the threshold and draws; the list holds every key >= its smallest one
     if (wave == 0) {
-      ListPass pass{list_val, list_idx, n_list, mx, invT};
-      unsigned long long lo_key = ~0ull;
-      for (int j = lane; j < n_list; j += 64) {
-        const unsigned long long k = key_of(list_val[j], list_idx[j]);
-        lo_key = k < lo_key ? k : lo_key;
-      }
-      for (int off = 32; off > 0; off >>= 1) {
-        const unsigned long long o = shfl_xor_u64(lo_key, off);
-        lo_key = o < lo_key ? o : lo_key;
-      }
-      const unsigned long long theta = find_theta(pass, best, lo_key >> 32, k_limit, e_floor, use_p, p_mass);
-      // the draw: running sum over the kept entries in index order, a contiguous run of the list a lane
-      const int chunk = (n_list + 63) / 64;
-      const int j0 = min(n_list, lane * chunk), j1 = min(n_list, j0 + chunk);
-      double mine = 0.0;
-      int cnt = 0;
-      for (int j = j0; j < j1; ++j)
-        if (key_of(list_val[j], list_idx[j]) >= theta) {
-          mine += (double)expf((list_val[j] - mx) * invT);
-          ++cnt;
-        }
-      double incl = mine;
-      for (int off = 1; off < 64; off <<= 1) {
-        const unsigned long long bits = (unsigned long long)__double_as_longlong(incl);
-        const unsigned hi32 = __shfl_up((unsigned)(bits >> 32), off, 64);
-        const unsigned lo32 = __shfl_up((unsigned)bits, off, 64);
-        const double o = __longlong_as_double((long long)(((unsigned long long)hi32 << 32) | lo32));
-        if (lane >= off) incl += o;
-      }
-      const double all = shfl_f64(incl, 63);  // the mass of the kept set
-      int kept = cnt;
-      for (int off = 32; off > 0; off >>= 1) kept += __shfl_xor(kept, off, 64);
-      const double r = u * all;
-      const double lo_excl = incl - mine;
-      int tok = -1;
-      if (cnt > 0 && r >= lo_excl && r < incl) {
-        double acc = lo_excl;
-        for (int j = j0; j < j1; ++j)
-          if (key_of(list_val[j], list_idx[j]) >= theta) {
-            acc += (double)expf((list_val[j] - mx) * invT);
-            tok = list_idx[j];
-            if (r < acc) break;
-          }
-      }
-      // at most one lane's range holds r
-      for (int off = 32; off > 0; off >>= 1) tok = max(tok, __shfl_xor(tok, off, 64));
+      const ListResult res = list_threshold_and_draw(list_val, list_idx, n_list, best, mx, invT, k_limit, e_floor, use_p,
+                                                     p_mass, u);
       if (lane == 0) {
-        tok_sh = tok;
-        kept_sh = kept;
-        total_sh = all;
+        tok_sh = res.tok;
+        kept_sh = res.kept;
+        total_sh = res.mass;
       }
     }
     __syncthreads();
@@ -736,6 +803,342 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(SampleArgs a) {
   }
 }
 
+// ------------------------------------------------------------------ top-k in parts
+// With a small top_k the kept set lies among the k largest of the row, and those lie among the k largest
+// of every slice of the row.  So the row is first cut into SAMPLE_PARTS slices, a block each: it leaves
+// its slice's largest key, the slice's sum of exp((l - slice max) / T), and the entries that rank among
+// the slice's k largest values (all that tie with the k-th: at most PART_CAP, else the row is flagged
+// and goes the long way), in index order.  One block a row then puts the parts together: the row's
+// maximum, Z = sum over the slices of their sums scaled to it, the list, and on it the same threshold
+// search and draw as above.  Five passes of one compute unit over the row become one pass of 32.
+constexpr int SAMPLE_PARTS = 32;
+constexpr int PART_THREADS = 256;
+constexpr int PART_PER_LANE = 16;                                     // a block takes up to 4096 entries
+constexpr int PART_MAX_SLICE = PART_THREADS * PART_PER_LANE;
+constexpr int PART_CAP = 96;                                          // entries a part may leave
+constexpr int PART_MAX_K = 64;
+constexpr int WAVE_CAP = 128;                                         // entries a wave may hand to its block
+
+struct PartOut {          // what a part leaves, rows x SAMPLE_PARTS of each
+  unsigned long long* best;  // largest key of the slice (BAD_ROW: a NaN or an infinity)
+  double* z;                 // sum of exp((l - slice max) / T)
+  int* count;                // entries left, or -1: more than PART_CAP rank with the k largest
+  float* val;                // [PART_CAP]
+  int* idx;                  // [PART_CAP]
+};
+
+__device__ inline PartOut part_out(unsigned char* scratch, int rows) {
+  const long long n = (long long)rows * SAMPLE_PARTS;
+  PartOut o;
+  o.best = (unsigned long long*)scratch;
+  o.z = (double*)(o.best + n);
+  o.val = (float*)(o.z + n);
+  o.idx = (int*)(o.val + n * PART_CAP);
+  o.count = o.idx + n * PART_CAP;
+  return o;
+}
+static long long part_scratch_bytes(int rows) {
+  return (long long)rows * SAMPLE_PARTS * (8 + 8 + 4 + PART_CAP * 8);
+}
+
+// A value v with at least k and at most `cap` of a wave's ordered-bit values >= v (a lane's PER of them
+// in registers); if no value cuts that finely (ties), the largest v with at least k values >= v, whatever
+// their number; with fewer than k values: 0.  The k largest are among the values >= v either way.
+template <int PER>
+__device__ inline unsigned cut_for_k_largest(const unsigned (&bits)[PER], int k, int cap) {
+  unsigned lo = 0u, hi = 0xffffffffu;  // count(>= lo) >= k holds for lo = 0 (if there are k at all)
+  while (lo < hi) {
+    const unsigned mid = lo + (hi - lo) / 2u + 1u;  // upper middle: lo < mid <= hi
+    int c = 0;  // counted with ballots: no lane waits for another
+#pragma unroll
+    for (int j = 0; j < PER; ++j) c += __popcll(__ballot(bits[j] >= mid));
+    if (c >= k) {
+      lo = mid;
+      if (c <= cap) break;
+    } else {
+      hi = mid - 1u;
+    }
+  }
+  return lo;
+}
+
+__global__ __launch_bounds__(PART_THREADS) void sample_parts_kernel(const float* __restrict__ logits, int ld, int V,
+                                                                    float invT, int top_k, unsigned char* scratch) {
+  __shared__ float wv[PART_THREADS / 64][WAVE_CAP];
+  __shared__ int wi[PART_THREADS / 64][WAVE_CAP];
+  __shared__ int wn[PART_THREADS / 64];
+  __shared__ unsigned long long wbest[PART_THREADS / 64];
+  __shared__ double wz[PART_THREADS / 64];
+  const int part = blockIdx.x, row = blockIdx.y, rows = gridDim.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const PartOut o = part_out(scratch, rows);
+  const long long at = (long long)row * SAMPLE_PARTS + part;
+  const int per = (V + SAMPLE_PARTS - 1) / SAMPLE_PARTS;
+  const int i0 = part * per, i1 = min(V, i0 + per);
+  const float* lr = logits + (long long)row * ld;
+  // a wave takes 1024 consecutive entries, 64 at a time (entry j of lane l: 64 j + l), so that loads are
+  // whole lines and (j, lane) order is index order
+  float v[PART_PER_LANE];
+  unsigned bits[PART_PER_LANE];
+  unsigned long long best = 0ull;
+  const int mine0 = i0 + wave * (64 * PART_PER_LANE) + lane;
+#pragma unroll
+  for (int j = 0; j < PART_PER_LANE; ++j) {
+    const int i = mine0 + 64 * j;
+    const bool has = i < i1;
+    v[j] = has ? lr[i] : 0.f;
+    bits[j] = has ? ordered_bits(v[j]) : 0u;  // (0 ranks below every number)
+    if (has) {
+      const unsigned long long k = checked_key_of(v[j], i);
+      best = k > best ? k : best;
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned long long ob = shfl_xor_u64(best, off);
+    best = ob > best ? ob : best;
+  }
+  if (lane == 0) wbest[wave] = best;
+  __syncthreads();
+  best = wbest[0];
+  for (int w = 1; w < PART_THREADS / 64; ++w) best = wbest[w] > best ? wbest[w] : best;
+  if (best == BAD_ROW || i0 >= i1) {  // the same for every thread of the block
+    if (tid == 0) {
+      o.best[at] = i0 >= i1 ? 0ull : BAD_ROW;
+      o.z[at] = 0.0;
+      o.count[at] = 0;
+    }
+    return;
+  }
+  const float mx = from_ordered_bits((unsigned)(best >> 32));
+  double z = 0.0;
+#pragma unroll
+  for (int j = 0; j < PART_PER_LANE; ++j)
+    if (mine0 + 64 * j < i1) z += (double)expf((v[j] - mx) * invT);
+  for (int off = 32; off > 0; off >>= 1) z += shfl_xor_f64(z, off);
+  if (lane == 0) wz[wave] = z;
+  // every wave: the entries that rank with its k largest values, to LDS in index order
+  const unsigned cut = cut_for_k_largest<PART_PER_LANE>(bits, top_k, WAVE_CAP);
+  const unsigned long long before = (1ull << lane) - 1ull;
+  int total = 0;
+  bool fits = true;
+#pragma unroll
+  for (int j = 0; j < PART_PER_LANE; ++j) {
+    const bool take = mine0 + 64 * j < i1 && bits[j] >= cut;
+    const unsigned long long m = __ballot(take);
+    const int pos = total + __popcll(m & before);
+    total += __popcll(m);
+    fits = fits && total <= WAVE_CAP;
+    if (take && fits) {
+      wv[wave][pos] = v[j];
+      wi[wave][pos] = mine0 + 64 * j;
+    }
+  }
+  if (lane == 0) wn[wave] = fits ? total : -1;
+  __syncthreads();
+  // wave 0: the k largest values among what the four waves left, again with their ties
+  if (wave != 0) return;
+  double zsum = 0.0;
+  bool over = false;
+  int n_all = 0;
+  for (int w = 0; w < PART_THREADS / 64; ++w) {
+    zsum += wz[w];
+    over = over || wn[w] < 0;
+    n_all += max(wn[w], 0);
+  }
+  if (lane == 0) {
+    o.best[at] = best;
+    o.z[at] = zsum;
+  }
+  if (over) {
+    if (lane == 0) o.count[at] = -1;
+    return;
+  }
+  // the waves' lists one after the other are in index order; a lane takes a run of 8 of them
+  constexpr int RUN = PART_THREADS / 64 * WAVE_CAP / 64;  // 8
+  float cv[RUN];
+  int ci[RUN];
+  unsigned cb[RUN];
+#pragma unroll
+  for (int j = 0; j < RUN; ++j) {
+    int q = lane * RUN + j;  // place in the concatenation
+    int w = 0;
+    while (w < PART_THREADS / 64 - 1 && q >= wn[w]) {
+      q -= wn[w];
+      ++w;
+    }
+    const bool has = lane * RUN + j < n_all;
+    cv[j] = has ? wv[w][q] : 0.f;
+    ci[j] = has ? wi[w][q] : -1;
+    cb[j] = has ? ordered_bits(cv[j]) : 0u;
+  }
+  const unsigned cut2 = cut_for_k_largest<RUN>(cb, top_k, PART_CAP);
+  int take2 = 0;
+#pragma unroll
+  for (int j = 0; j < RUN; ++j) take2 += (ci[j] >= 0 && cb[j] >= cut2) ? 1 : 0;
+  int incl2 = take2;
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(incl2, off, 64);
+    if (lane >= off) incl2 += up;
+  }
+  const int total2 = __shfl(incl2, 63, 64);
+  if (total2 <= PART_CAP) {
+    int pos = incl2 - take2;
+#pragma unroll
+    for (int j = 0; j < RUN; ++j)
+      if (ci[j] >= 0 && cb[j] >= cut2) {
+        o.val[at * PART_CAP + pos] = cv[j];
+        o.idx[at * PART_CAP + pos] = ci[j];
+        ++pos;
+      }
+  }
+  if (lane == 0) o.count[at] = total2 <= PART_CAP ? total2 : -1;
+}
+
+// One block a row: puts the parts together and draws.  Rows whose parts were flagged are left for the
+// long way (redo[row] = 1), which the host launches over all rows right after: it skips the others.
+__global__ __launch_bounds__(256) void sample_merge_kernel(SampleArgs a, const unsigned char* scratch, int* redo) {
+  __shared__ float list_val[SAMPLE_PARTS * PART_CAP];
+  __shared__ int list_idx[SAMPLE_PARTS * PART_CAP];
+  __shared__ int offset[SAMPLE_PARTS + 1];
+  __shared__ unsigned long long key_sh[4 * PART_MAX_K];
+  __shared__ float e_sh[4 * PART_MAX_K];
+  __shared__ unsigned long long best_sh;
+  __shared__ double z_sh;
+  __shared__ int floor_count;
+  const int row = blockIdx.x, rows = gridDim.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const PartOut o = part_out(const_cast<unsigned char*>(scratch), rows);
+  const long long at0 = (long long)row * SAMPLE_PARTS;
+  const float invT = a.inv_temperature;
+  if (wave == 0) {
+    // the row's maximum, the flags, the places of the parts' lists
+    unsigned long long best = lane < SAMPLE_PARTS ? o.best[at0 + lane] : 0ull;
+    int cnt = lane < SAMPLE_PARTS ? o.count[at0 + lane] : 0;
+    int flagged = cnt < 0 ? 1 : 0;
+    for (int off = 32; off > 0; off >>= 1) {
+      const unsigned long long ob = shfl_xor_u64(best, off);
+      best = ob > best ? ob : best;
+      flagged |= __shfl_xor(flagged, off, 64);
+    }
+    int incl = max(cnt, 0);
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += up;
+    }
+    if (lane < SAMPLE_PARTS) offset[lane + 1] = incl;
+    if (lane == 0) offset[0] = 0;
+    // Z = sum over the parts of z_p * exp((m_p - m) / T), in part order
+    const float mx = from_ordered_bits((unsigned)(best >> 32));
+    double term = 0.0;
+    if (lane < SAMPLE_PARTS && best != BAD_ROW && o.best[at0 + lane] != 0ull) {
+      const float mp = from_ordered_bits((unsigned)(o.best[at0 + lane] >> 32));
+      term = o.z[at0 + lane] * exp(((double)mp - (double)mx) * (double)invT);
+    }
+    double zsum = 0.0;
+    for (int p = 0; p < SAMPLE_PARTS; ++p) zsum += shfl_f64(term, p);
+    if (lane == 0) {
+      best_sh = flagged && best != BAD_ROW ? 1ull : best;  // 1: the long way
+      z_sh = zsum;
+      floor_count = 0;
+    }
+  }
+  __syncthreads();
+  const unsigned long long best = best_sh;
+  if (best == BAD_ROW || best == 1ull) {
+    if (tid == 0) {
+      if (best == BAD_ROW) {
+        a.out[row] = NO_TOKEN;
+        if (a.kept_count) a.kept_count[row] = 0;
+        if (a.kept_mass) a.kept_mass[row] = 0.0;
+        redo[row] = 0;
+      } else {
+        redo[row] = 1;
+      }
+    }
+    return;
+  }
+  const float mx = from_ordered_bits((unsigned)(best >> 32));
+  const double Z = z_sh;
+  const double e_floor = 1e-10 * Z;
+  const bool use_p = a.top_p > 0.f && a.top_p < 1.f;
+  const double p_mass = (double)a.top_p * Z;
+  const int n_list = offset[SAMPLE_PARTS];
+  int above = 0;
+  // every thread asks for its entries of the list at once: which part an entry belongs to is looked up
+  // in the parts' offsets (the loads of all parts are then in flight together)
+  for (int j = tid; j < n_list; j += 256) {
+    int p = 0;
+#pragma unroll
+    for (int step = SAMPLE_PARTS / 2; step > 0; step >>= 1)
+      if (offset[p + step] <= j) p += step;
+    const long long src = (at0 + p) * PART_CAP + (j - offset[p]);
+    const float v = o.val[src];
+    list_val[j] = v;
+    list_idx[j] = o.idx[src];
+    above += (double)expf((v - mx) * invT) > e_floor ? 1 : 0;
+  }
+  for (int off = 32; off > 0; off >>= 1) above += __shfl_xor(above, off, 64);
+  if (lane == 0) atomicAdd(&floor_count, above);
+  __syncthreads();
+  if (wave != 0) return;
+  // every candidate of the row (p > 1e-10) that ranks among the k largest is in the list; if the row has
+  // fewer than k candidates, all of them are
+  const long long k_limit = min((long long)a.top_k, (long long)floor_count);
+  // the list is 32 times what is needed: keep what ranks with its k largest values (a coarse cut by
+  // counting alone), in place and in order, and search that
+  int n_short = n_list;
+  {
+    constexpr int PER = SAMPLE_PARTS * PART_CAP / 64;  // 48
+    // entry j of lane l is 64 j + l: neighbouring lanes read neighbouring words, and (j, lane) order is
+    // index order.  Everything is read before anything is written, and an entry moves to its own place or
+    // one before it.
+    float mv[PER];
+    int mi[PER];
+    unsigned lb[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const bool has = 64 * j + lane < n_list;
+      mv[j] = has ? list_val[64 * j + lane] : 0.f;
+      mi[j] = has ? list_idx[64 * j + lane] : -1;
+      lb[j] = has ? ordered_bits(mv[j]) : 0u;
+    }
+    const unsigned cut = cut_for_k_largest<PER>(lb, a.top_k, 4 * PART_MAX_K);
+    const unsigned long long before = (1ull << lane) - 1ull;
+    int total = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const bool take = mi[j] >= 0 && lb[j] >= cut;
+      const unsigned long long m = __ballot(take);
+      if (take) {
+        const int pos = total + __popcll(m & before);
+        list_val[pos] = mv[j];
+        list_idx[pos] = mi[j];
+      }
+      total += __popcll(m);
+    }
+    n_short = total;
+  }
+  const int slot = a.seq_slot[row];
+  const unsigned long long ctr = (unsigned long long)a.rng_ctr[slot];
+  const double u = uniform_of((unsigned long long)a.rng_key[slot], ctr);
+  ListResult res;
+  if (n_short <= 4 * PART_MAX_K)
+    res = list_draw(list_val, list_idx, n_short,
+                    list_threshold_by_ranks(list_val, list_idx, n_short, mx, invT, k_limit, e_floor, use_p, p_mass, key_sh, e_sh), mx,
+                    invT, u);
+  else  // (ties beyond what the coarse cut could separate)
+    res = list_threshold_and_draw(list_val, list_idx, n_short, best, mx, invT, k_limit, e_floor, use_p, p_mass, u);
+  if (lane == 0) {
+    int tok = res.tok;
+    if (tok < 0) tok = (int)(0xffffffffu - (unsigned)(best & 0xffffffffull));  // r fell on a rounding seam
+    a.out[row] = tok;
+    a.rng_ctr[slot] = (long long)(ctr + 1ull);
+    if (a.recent) push_recent(a.recent, a.recent_n, slot, tok);
+    if (a.kept_count) a.kept_count[row] = res.kept;
+    if (a.kept_mass) a.kept_mass[row] = res.mass / Z;
+    redo[row] = 0;
+  }
+}
+
 // ------------------------------------------------------------------ state upkeep
 __global__ void advance_kernel(int* row_pos, int* seq_start, int* seq_len, int batch) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -813,12 +1216,18 @@ extern "C" int lq_argmax_no_alloc(const float* logits, int ld, int rows, int V, 
   return 0;
 }
 
+// Bytes of scratch with which lq_sample takes the short way for `rows` rows (top_k in 1..64 and a
+// vocabulary of 8 192 to 131 072 entries); without it, or outside these sizes, it goes the long way.
+extern "C" long long lq_sample_scratch_bytes(int rows) { return part_scratch_bytes(rows) + (long long)rows * 4; }
+
 extern "C" int lq_sample(const float* logits, int ld, int rows, int V, const int* seq_slot, float temperature,
                          int top_k, float top_p, long long* rng_key, long long* rng_ctr, int* recent,
-                         int* recent_n, int* out, int* kept_count, double* kept_mass, hipStream_t stream) {
+                         int* recent_n, int* out, int* kept_count, double* kept_mass, void* scratch,
+                         long long scratch_bytes, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && V > 0 && ld >= V, "sample: bad sizes");
   LQ_REQUIRE(temperature > 0.f, "sample: temperature %f must be positive (0 is the greedy kernel)", temperature);
   LQ_REQUIRE(seq_slot && rng_key && rng_ctr && out, "sample: null pointer");
+  LQ_REQUIRE(rows <= 65535, "sample: %d rows are too many for one launch", rows);
   SampleArgs a;
   a.logits = logits;
   a.ld = ld;
@@ -834,7 +1243,21 @@ extern "C" int lq_sample(const float* logits, int ld, int rows, int V, const int
   a.out = out;
   a.kept_count = kept_count;
   a.kept_mass = kept_mass;
-  sample_kernel<<<rows, THREADS, 0, stream>>>(a);
+  const bool parts = scratch != nullptr && scratch_bytes >= lq_sample_scratch_bytes(rows) && top_k >= 1 &&
+                     top_k <= PART_MAX_K && V >= 8192 && V <= SAMPLE_PARTS * PART_MAX_SLICE &&
+                     ((uintptr_t)scratch % 8) == 0;
+  if (!parts) {
+    sample_kernel<<<rows, THREADS, 0, stream>>>(a, nullptr);
+    LQ_CHECK_LAUNCH("sample");
+    return 0;
+  }
+  int* redo = (int*)((unsigned char*)scratch + part_scratch_bytes(rows));
+  sample_parts_kernel<<<dim3(SAMPLE_PARTS, rows), PART_THREADS, 0, stream>>>(logits, ld, V, a.inv_temperature, top_k,
+                                                                            (unsigned char*)scratch);
+  sample_merge_kernel<<<rows, 256, 0, stream>>>(a, (const unsigned char*)scratch, redo);
+  // rows with more ties at a slice's k-th value than a part can hold (redo = 1): the long way, the others
+  // leave at once
+  sample_kernel<<<rows, THREADS, 0, stream>>>(a, redo);
   LQ_CHECK_LAUNCH("sample");
   return 0;
 }

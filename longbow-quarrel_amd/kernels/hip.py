@@ -488,9 +488,14 @@ class HipKernels:
     def sample(self, logits: torch.Tensor, out: torch.Tensor, seq_slot: torch.Tensor, temperature: float,
                top_k: int, top_p: float, rng_key: torch.Tensor, rng_ctr: torch.Tensor,
                recent: Optional[torch.Tensor] = None, recent_n: Optional[torch.Tensor] = None,
-               kept_count: Optional[torch.Tensor] = None, kept_mass: Optional[torch.Tensor] = None) -> None:
-        """Temperature sampling with top-k and top-p; each sequence's counter moves on by one."""
-        self._dev(logits, out, seq_slot, rng_key, rng_ctr, recent, recent_n, kept_count, kept_mass)
+               kept_count: Optional[torch.Tensor] = None, kept_mass: Optional[torch.Tensor] = None,
+               scratch: Optional[torch.Tensor] = None) -> None:
+        """Temperature sampling with top-k and top-p; each sequence's counter moves on by one.  With
+        `scratch` (uint8, `sample_scratch_bytes(rows)`) and a small top-k the row is worked on in parts
+        by many compute units instead of one."""
+        self._dev(logits, out, seq_slot, rng_key, rng_ctr, recent, recent_n, kept_count, kept_mass, scratch)
+        if scratch is not None and (scratch.dtype != torch.uint8 or not scratch.is_contiguous()):
+            raise KernelLibraryError("sample: scratch must be dense uint8")
         rows, vocab = logits.shape
         self._i32(out, "sample out", rows)
         self._i32(seq_slot, "seq_slot", rows)
@@ -503,7 +508,13 @@ class HipKernels:
         self._check(self.lib.lq_sample(_ptr(logits), c_int(self._rows2d(logits, "logits")), c_int(rows),
                                        c_int(vocab), _ptr(seq_slot), c_float(temperature), c_int(top_k),
                                        c_float(top_p), _ptr(rng_key), _ptr(rng_ctr), _ptr(recent), _ptr(recent_n),
-                                       _ptr(out), _ptr(kept_count), _ptr(kept_mass), self.stream))
+                                       _ptr(out), _ptr(kept_count), _ptr(kept_mass), _ptr(scratch),
+                                       c_longlong(scratch.numel() if scratch is not None else 0), self.stream))
+
+    @query
+    def sample_scratch_bytes(self, rows: int) -> int:
+        self.lib.lq_sample_scratch_bytes.restype = c_longlong
+        return int(self.lib.lq_sample_scratch_bytes(c_int(rows)))
 
     def advance(self, row_pos: torch.Tensor, seq_start: torch.Tensor, seq_len: torch.Tensor, batch: int) -> None:
         """Positions and lengths of a decoding batch move on by one."""

@@ -24,6 +24,8 @@ class Sampler:
         self.kernels = kernels
         self.state = state
         self.params = params
+        # made now, not inside a step: a captured step must not allocate
+        self.scratch = None if params.greedy else state.scratch_for_sampling(kernels, state.rng_key.numel())
 
     def sample(self, logits: torch.Tensor, seq_slot: torch.Tensor, out: torch.Tensor) -> None:
         """logits float32 [batch, vocab] (changed in place by the penalty), seq_slot int32 [batch],
@@ -35,7 +37,7 @@ class Sampler:
             kn.argmax(logits, out, st.argmax_scratch, seq_slot, st.recent, st.recent_n)
         else:
             kn.sample(logits, out, seq_slot, p.temperature, p.top_k, p.top_p, st.rng_key, st.rng_ctr,
-                      st.recent, st.recent_n)
+                      st.recent, st.recent_n, scratch=self.scratch)
 
     @staticmethod
     def read_tokens(out: torch.Tensor) -> List[int]:

@@ -31,6 +31,16 @@ class SamplerState:
         self.recent_n = torch.zeros(max_slots, dtype=torch.int32, device=device)
         # what the two stages of the arg-max kernel pass between them: 32 words for each row of a batch
         self.argmax_scratch = torch.zeros(32 * max_slots, dtype=torch.int64, device=device)
+        # what the stages of temperature sampling with a small top-k pass between them (made when first asked for)
+        self.sample_scratch = None
+
+    def scratch_for_sampling(self, kernels, rows: int):
+        need = getattr(kernels, "sample_scratch_bytes", None)
+        if need is None:
+            return None
+        if self.sample_scratch is None:
+            self.sample_scratch = torch.zeros(need(self.rng_key.numel()), dtype=torch.uint8, device=self.device)
+        return self.sample_scratch if rows <= self.rng_key.numel() else None
 
     def start(self, slot: int, key: int, history: Sequence[int]) -> None:
         """A sequence starts in `slot`: generator at draw 0, ring holding the end of its prompt."""

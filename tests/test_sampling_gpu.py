@@ -42,7 +42,7 @@ def draw_in_index_order(dist, u):
     return last
 
 
-def run(kn, logits, params, slots=None, state=None, history=None):
+def run(kn, logits, params, slots=None, state=None, history=None, parts=False):
     rows, vocab = logits.shape
     slots = slots or list(range(rows))
     state = state or SamplerState(max(slots) + 1, DEV)
@@ -59,8 +59,9 @@ def run(kn, logits, params, slots=None, state=None, history=None):
     if params.greedy:
         kn.argmax(lg, out, state.argmax_scratch, seq_slot, state.recent, state.recent_n)
     else:
+        scratch = torch.empty(kn.sample_scratch_bytes(rows), dtype=torch.uint8, device=DEV) if parts else None
         kn.sample(lg, out, seq_slot, params.temperature, params.top_k, params.top_p, state.rng_key, state.rng_ctr,
-                  state.recent, state.recent_n, kept, mass)
+                  state.recent, state.recent_n, kept, mass, scratch=scratch)
     return out.cpu().tolist(), kept.cpu().tolist(), mass.cpu().tolist(), state, lg.cpu()
 
 
@@ -104,6 +105,49 @@ def test_kept_set_and_draw_follow_the_plain_sampler(kn, vocab, temperature, top_
         assert tok[r] == draw_in_index_order(dist, u)
         assert tok[r] in dist
     assert state.rng_ctr.cpu().tolist()[:6] == [1, 0, 1, 1, 0, 1]  # each sampled sequence moved on by one draw
+
+
+@pytest.mark.parametrize("vocab", [8192, 50021, 128256, 131072])
+@pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, 40, 1.0), (0.7, 40, 0.95), (1.3, 5, 0.5), (0.8, 1, 1.0),
+                                                    (0.5, 64, 0.999), (2.0, 17, 0.3)])
+def test_a_small_top_k_worked_on_in_parts_gives_what_the_one_block_kernel_and_the_plain_sampler_give(
+        kn, vocab, temperature, top_k, top_p):
+    """With scratch memory and top_k <= 64 the row is cut into 32 slices that leave their k largest; the
+    kept set, the draw and the generator's counter are those of the kernel that walks the row alone."""
+    g = torch.Generator().manual_seed(vocab + top_k)
+    logits = torch.randn((5, vocab), generator=g) * 3.0
+    logits[3] = (logits[3] * 2).round() / 2  # half-integer logits: many ties, in every slice
+    logits[4, :] = -5.0
+    logits[4, [3, vocab // 2, vocab - 1]] = torch.tensor([1.0, 1.5, 0.5])  # a peaked row: fewer candidates than k
+    params = SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p, seed=11)
+    slots = [3, 0, 2, 5, 1]
+    alone = run(kn, logits, params, slots=slots, history=[[1]] * 5)
+    parts = run(kn, logits, params, slots=slots, history=[[1]] * 5, parts=True)
+    assert parts[0] == alone[0] and parts[1] == alone[1]
+    assert max(abs(a - b) for a, b in zip(parts[2], alone[2])) < 1e-6
+    assert parts[3].rng_ctr.cpu().tolist() == alone[3].rng_ctr.cpu().tolist()
+    assert parts[3].recent_n.cpu().tolist() == alone[3].recent_n.cpu().tolist()
+    for r in (0, 1, 2, 4):
+        dist = plain.candidate_distribution(logits[r], temperature, top_k, top_p)
+        assert parts[1][r] == len(dist) and parts[0][r] in dist
+        u = uniform_of(sequence_key(11, slots[r]) & MASK, 0)
+        assert parts[0][r] == draw_in_index_order(dist, u)
+
+
+def test_rows_with_more_ties_than_a_part_holds_go_the_long_way(kn):
+    """A row of equal logits: every slice's k-th value ties with thousands, no part can hold them, and the
+    row is sampled by the kernel that walks it alone; the row beside it goes through the parts."""
+    vocab = 128256
+    g = torch.Generator().manual_seed(9)
+    logits = torch.randn((3, vocab), generator=g)
+    logits[1] = 0.25
+    logits[2, 1000:] = float("nan")
+    params = SamplingParams(temperature=0.9, top_k=40, top_p=0.9, seed=4)
+    alone = run(kn, logits, params, history=[[1]] * 3)
+    parts = run(kn, logits, params, history=[[1]] * 3, parts=True)
+    assert parts[0] == alone[0] and parts[1] == alone[1] and parts[0][2] == -1
+    assert parts[1][1] == 40 and 0 <= parts[0][1] < 40  # the first 40 indices of the tie, in index order
+    assert parts[3].rng_ctr.cpu().tolist() == alone[3].rng_ctr.cpu().tolist() == [1, 1, 0]
 
 
 def test_ties_are_kept_in_index_order(kn):
