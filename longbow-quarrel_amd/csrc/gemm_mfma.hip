@@ -68,7 +68,14 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
 // row, the sum of squares of the block's updated columns in a table, for the norm that follows.
 enum { EPI_NONE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 2 };
 
-__device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+// silu(g) u = g u / (1 + e^-g), for 16-bit outputs: the hardware's exponential and reciprocal (an ulp or so
+// each, far below the rounding of the result) instead of a division and a library call per element
+__device__ inline float silu_mul(float g, float u) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u; }
+
+// the value of the lane 8 places away within its row of 16 lanes (lane ^ 8), by a DPP rotation
+__device__ inline float from_lane_xor8(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, true));
+}
 
 // A wave's WM x WN accumulators of 32 x 32 go to C (rows from row0, columns from col0).
 template <int WM, int WN, int EPI, typename TO>
@@ -107,13 +114,23 @@ __device__ inline void block_epilogue_16(f32x16 (&acc)[WM][WN], bf16_t* __restri
 #pragma unroll
     for (int j = 0; j < WN; ++j) {
       const int col = wcol + j * 32 + (lane & 31);  // within the block tile
+      if constexpr (EPI == EPI_SWIGLU) {
+        // Gate column c (c % 16 < 8) and its up column c + 8 sit 8 lanes apart.  Two rows at a time: the
+        // gate lane takes the up value of the first row from its partner and gives it the gate value of the
+        // second, so that every lane works out one product of the pair and no lane stands idle.
+        const bool gate_lane = (lane & 8) == 0;
+        const int out_col = ((col >> 4) << 3) + (col & 7);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = wrow + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (EPI == EPI_SWIGLU) {
-          const float up = __shfl(acc[i][j][e], lane + 8, 64);
-          if ((col & 15) < 8) tile[row * OUT_W + ((col >> 4) << 3) + (col & 7)] = f32_to_bf16(silu_mul(acc[i][j][e], up));
-        } else {
+        for (int e = 0; e < 16; e += 2) {
+          const int row = wrow + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3) + (gate_lane ? 0 : 1);
+          const float got = from_lane_xor8(gate_lane ? acc[i][j][e + 1] : acc[i][j][e]);
+          const float v = gate_lane ? silu_mul(acc[i][j][e], got) : silu_mul(got, acc[i][j][e + 1]);
+          tile[row * OUT_W + out_col] = f32_to_bf16(v);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = wrow + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
           tile[row * OUT_W + col] = f32_to_bf16(acc[i][j][e]);
         }
       }
@@ -405,26 +422,54 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     // slab t, the other reads its fragments of slab t (or t + 1) from LDS, so the matrix pipe and the LDS
     // port of a SIMD work at the same time.  Every wave runs  fetch(t) | barrier | multiply(t) | barrier;
     // the second group has passed one barrier more before it starts, which puts it half a period behind.
-    // Who may overwrite what: slab t is read by group 0 before its barrier X(t) and by group 1 before its
-    // X'(t), which is group 0's Y(t).  So after Y(t) (group 0: start of fetch(t + 1); group 1: start of
-    // multiply(t)) both ask for slab t + 2 into slab t's stage, and both wait for their own transfers of
-    // it two phases later, before the barrier that precedes the first read of slab t + 2 (group 0: end of
-    // multiply(t + 1); group 1: end of fetch(t + 1)).
-    static_assert(!ALTERNATE || (STAGES == 2 && S::NW == 8), "two stages, two groups of four waves");
-    const int group = wave >> 2;
-    dma(0, 0);
-    if (slabs > 1) {
-      dma(1, BK);
-      LQ_WAIT_VMCNT(S::DMA);
-    } else {
+    static_assert(!ALTERNATE || (STAGES == 2 && GM == 4 && GN == 2), "two stages, two groups of four waves");
+    // Transfers are asked for in the fetch phases, after the wave's fragment reads are on their way: there
+    // they cost nothing, while a wave that asks between its products (or before its reads) holds up the
+    // matrix pipe (or the barrier) for as long as the address unit takes.  Group 0's waves fetch W, group 1's
+    // fetch A, a wave every fourth transfer of its operand.  What may be overwritten when (stage s = t % 2
+    // holds slab t; group 0 reads slab t + 1 while group 1 multiplies slab t; group 1 reads slab t + 1 while
+    // group 0 multiplies it):
+    //   W of slab t + 1, by group 0 after its reads of slab t: everyone has read W of slab t - 1 (group 1 last,
+    //     before it multiplied slab t - 1, which it does now);
+    //   group 1's own A rows of slab t + 1, by group 1 after its reads of slab t: it read those of slab t - 1 a
+    //     period ago;
+    //   group 0's A rows of slab t + 2, by group 1 at the same time, into the stage it is reading: group 0 has
+    //     read its rows of slab t and multiplies them now.
+    // Addresses: a buffer descriptor over the tile's valid rows (rows past the matrix read as zeros, no
+    // clamping by hand), a lane offset (row within a transfer, swizzled chunk), the transfer's rows added to
+    // it, and the slab's k as the scalar offset.
+    const int group = wave >> 2, w4 = wave & 3;
+    static_assert(S::BM == S::BN, "as many transfers of A as of W");
+    constexpr int NT = S::BM / S::ROWS_PER_DMA / 4;  // a wave's transfers of a slab
+    static_assert(S::BM % (S::ROWS_PER_DMA * 8) == 0, "whole transfers for four waves, half of them group 0's A rows");
+    static_assert((4 * S::ROWS_PER_DMA) % ((256 / S::ROW_BYTES) * S::CPR) == 0, "a wave's transfers lie whole swizzle periods apart");
+    const int lrow = lane / S::CPR;
+    const int lchunk = ((lane % S::CPR) ^ S::swizzle(w4 * S::ROWS_PER_DMA + lrow)) * 16;
+    const int ld = group == 0 ? ldw : lda;
+    const int t_voff = (w4 * S::ROWS_PER_DMA + lrow) * ld * 2 + lchunk;  // this lane in the wave's transfer 0
+    const int t_step = 4 * S::ROWS_PER_DMA * ld * 2;                      // to the wave's next transfer
+    const __amdgpu_buffer_rsrc_t t_rsrc =
+        group == 0 ? __builtin_amdgcn_make_buffer_rsrc((void*)w_origin, 0, min(N - n0, S::BN) * ldw * 2, 0x00020000)
+                   : __builtin_amdgcn_make_buffer_rsrc((void*)a_origin, 0, min(M - m0, S::BM) * lda * 2, 0x00020000);
+    const int t_dst = (group == 0 ? S::A_BYTES : 0) + w4 * 1024;  // in a stage; 4 KiB on a transfer
+    auto transfer = [&](int j, int stage, int k0) {
+      int v = t_voff;
+      asm volatile("" : "+v"(v));  // added up anew every time: kept across the loop it would cost a register a transfer
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(t_rsrc, LQ_LDS_PTR(plds + stage * S::STAGE_BYTES + t_dst + j * 4096), 16,
+                                               v + j * t_step, k0 * 2, 0, 0);
+    };
+    for (int q = 0; q < 2 && q < slabs; ++q)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) transfer(j, q, q * BK);
+    if (slabs > 1)
+      LQ_WAIT_VMCNT(NT);
+    else
       LQ_WAIT_VMCNT(0);
-    }
     asm volatile("s_barrier" ::: "memory");             // slab 0 is there
     if (group == 1) asm volatile("s_barrier" ::: "memory");  // half a period behind
     auto turn = [&](int stage, int t) {
       const unsigned char* as = a_base + stage * S::STAGE_BYTES;
       const unsigned char* ws = w_base + stage * S::STAGE_BYTES;
-      if (group == 0 && t >= 1 && t + 1 < slabs) dma(stage ^ 1, (t + 1) * BK);
       bf16x8 a[S::KK][WM], b[S::KK][WN];
 #pragma unroll
       for (int kk = 0; kk < S::KK; ++kk) {
@@ -433,12 +478,33 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
 #pragma unroll
         for (int j = 0; j < WN; ++j) b[kk][j] = as_bf16x8(*(const u32x4*)(ws + j * 32 * S::ROW_BYTES + frag[kk]));
       }
-      if (group == 1) LQ_WAIT_VMCNT(0);
+      const bool next = t >= 1 && t + 1 < slabs, after_next = t + 2 < slabs;
+      if (group == 0) {
+        if (next) {
+#pragma unroll
+          for (int j = 0; j < NT; ++j) transfer(j, stage ^ 1, (t + 1) * BK);  // W of slab t + 1
+        }
+      } else {
+        if (next) {
+#pragma unroll
+          for (int j = NT / 2; j < NT; ++j) transfer(j, stage ^ 1, (t + 1) * BK);  // own A rows of slab t + 1
+        }
+        if (after_next) {
+#pragma unroll
+          for (int j = 0; j < NT / 2; ++j) transfer(j, stage, (t + 2) * BK);  // group 0's A rows of slab t + 2
+        }
+        // group 0's A rows of slab t + 1, asked for a period ago, have landed: it reads them after the barrier
+        if (next && after_next)
+          LQ_WAIT_VMCNT(NT);
+        else if (next || after_next)
+          LQ_WAIT_VMCNT(NT / 2);
+        else
+          LQ_WAIT_VMCNT(0);
+      }
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the fragments are in registers
       __builtin_amdgcn_sched_barrier(0);
       asm volatile("s_barrier" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
-      if (group == 1 && t + 2 < slabs) dma(stage, (t + 2) * BK);
       __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int kk = 0; kk < S::KK; ++kk)
@@ -448,7 +514,12 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
           for (int j = 0; j < WN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_s_setprio(0);
-      if (group == 0) LQ_WAIT_VMCNT(0);
+      // what the next fetch phases read of slab t + 1 has landed: all of W (group 0's transfers), group 1's
+      // own A rows (asked for before group 0's rows of slab t + 2, which may still fly)
+      if (group == 0 || !after_next)
+        LQ_WAIT_VMCNT(0);
+      else
+        LQ_WAIT_VMCNT(NT / 2);
       __builtin_amdgcn_sched_barrier(0);
       asm volatile("s_barrier" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
