@@ -319,7 +319,19 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
   const int total = tiles_m * tiles_n;
   int pid = blockIdx.x;
   if (total % 8 == 0) pid = (pid % 8) * (total / 8) + pid / 8;  // one XCD walks a contiguous run of tiles
-  const int tm = pid % tiles_m, tn = pid / tiles_m;
+  int tm = pid % tiles_m, tn = pid / tiles_m;
+  if (total % 8 == 0 && tiles_m > 8 && (total / 8) % tiles_m == 0) {
+    // The 32 tiles that an XCD works on together should share operands both ways: 8 row tiles by 4 column
+    // tiles ask for 12 tiles' worth of operand rows, 32 row tiles of one column tile for 33.  The XCD's run
+    // is whole columns of tiles: walk them four columns at a time, and each such band in windows of 8 row
+    // tiles (the last window of a band has what is left).
+    const int run = total / 8, cols = run / tiles_m, r = pid % run, first_col = (pid / run) * cols;
+    const int band = r / (4 * tiles_m), in_band = r % (4 * tiles_m), width = min(4, cols - 4 * band);
+    const int whole = tiles_m / 8, window = min(in_band / (8 * width), whole);
+    const int in_window = in_band - window * 8 * width, height = window < whole ? 8 : tiles_m - 8 * whole;
+    tm = window * 8 + in_window % height;
+    tn = first_col + 4 * band + in_window / height;
+  }
   const int m0 = tm * S::BM, n0 = tn * S::BN;
   const int k_begin = blockIdx.y * k_share;
   C += blockIdx.y * split_stride;
