@@ -451,9 +451,10 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     // clamping by hand), a lane offset (row within a transfer, swizzled chunk), the transfer's rows added to
     // it, and the slab's k as the scalar offset.
     const int group = wave >> 2, w4 = wave & 3;
-    static_assert(S::BM == S::BN, "as many transfers of A as of W");
-    constexpr int NT = S::BM / S::ROWS_PER_DMA / 4;  // a wave's transfers of a slab
-    static_assert(S::BM % (S::ROWS_PER_DMA * 8) == 0, "whole transfers for four waves, half of them group 0's A rows");
+    constexpr int NT = S::BM / S::ROWS_PER_DMA / 4;    // a wave's transfers of a slab of A (group 1)
+    constexpr int NT_W = S::BN / S::ROWS_PER_DMA / 4;  // and of W (group 0)
+    static_assert(S::BM % (S::ROWS_PER_DMA * 8) == 0 && S::BN % (S::ROWS_PER_DMA * 4) == 0,
+                  "whole transfers for four waves, half of A group 0's rows");
     static_assert((4 * S::ROWS_PER_DMA) % ((256 / S::ROW_BYTES) * S::CPR) == 0, "a wave's transfers lie whole swizzle periods apart");
     const int lrow = lane / S::CPR;
     const int lchunk = ((lane % S::CPR) ^ S::swizzle(w4 * S::ROWS_PER_DMA + lrow)) * 16;
@@ -472,11 +473,14 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     };
     for (int q = 0; q < 2 && q < slabs; ++q)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) transfer(j, q, q * BK);
-    if (slabs > 1)
-      LQ_WAIT_VMCNT(NT);
-    else
+      for (int j = 0; j < (NT > NT_W ? NT : NT_W); ++j)
+        if (j < (group == 0 ? NT_W : NT)) transfer(j, q, q * BK);
+    if (slabs == 1)
       LQ_WAIT_VMCNT(0);
+    else if (group == 0)
+      LQ_WAIT_VMCNT(NT_W);
+    else
+      LQ_WAIT_VMCNT(NT);
     asm volatile("s_barrier" ::: "memory");             // slab 0 is there
     if (group == 1) asm volatile("s_barrier" ::: "memory");  // half a period behind
     auto turn = [&](int stage, int t) {
@@ -494,7 +498,7 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
       if (group == 0) {
         if (next) {
 #pragma unroll
-          for (int j = 0; j < NT; ++j) transfer(j, stage ^ 1, (t + 1) * BK);  // W of slab t + 1
+          for (int j = 0; j < NT_W; ++j) transfer(j, stage ^ 1, (t + 1) * BK);  // W of slab t + 1
         }
       } else {
         if (next) {
@@ -987,14 +991,16 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
     // Tiles run in rounds of one a compute unit; a narrower tile can save a round or fill a round that
     // a wider one leaves part empty.  Cost of a round relative to the 256-column tile, as measured.
     const int cus = lq_compute_units(), tm = lq_ceil_div(M, 256);
-    const double c256 = 1.00 * lq_ceil_div(tm * lq_ceil_div(N, 256), cus);
-    const double c224 = 1.02 * lq_ceil_div(tm * lq_ceil_div(N, 224), cus);
-    const double c192 = 0.83 * lq_ceil_div(tm * lq_ceil_div(N, 192), cus);
+    // (A last round that is part empty costs less than a whole one, which the rounding up does not know: a
+    // narrower tile has to win by a margin.)
+    const double c256 = 0.95 * lq_ceil_div(tm * lq_ceil_div(N, 256), cus);
+    const double c224 = 1.13 * lq_ceil_div(tm * lq_ceil_div(N, 224), cus);
+    const double c192 = 0.78 * lq_ceil_div(tm * lq_ceil_div(N, 192), cus);
     if (c256 <= c224 && c256 <= c192)
       return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     if (c224 <= c192)
       return launch_pipelined<8, 1, 1, 7, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
-    return launch_pipelined<4, 2, 2, 3, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    return launch_pipelined<4, 2, 2, 3, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
   }
   if (K % 32 == 0 && t128 >= lq_compute_units())
     return launch_pipelined<2, 2, 2, 4, 32, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
