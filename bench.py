@@ -127,11 +127,15 @@ def main() -> int:
             lens = torch.randint(prompt_len, args.prompt_len_max + 1, (batch,), generator=gen).tolist()
         prompts = [random_prompt(n) for n in lens]
         toks = backend.prefill(slots, prompts)  # in portions of at most 8,192 rows a step
-        for _ in range(warmup):
+        # as the generation loop does, the backend is told before the last step of a run that none follows: it
+        # queues no step ahead then, and exactly `steps` steps run between the two synchronisations
+        for i in range(warmup):
+            backend.expect_more(i + 1 < warmup)
             toks = backend.decode(slots, toks, False)
         torch.cuda.synchronize()
         t = time.perf_counter()
-        for _ in range(steps):
+        for i in range(steps):
+            backend.expect_more(i + 1 < steps)
             toks = backend.decode(slots, toks, False)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t

@@ -5,24 +5,27 @@
 
 // ---------------------------------------------------------------- embedding
 // out[r, :] = float(table[token[r], :])   (row copy, internal/device/kernels.metal:465-467)
+// A token that is no row of the table (a replayed step can be handed the sampler's "no token" before the
+// host has seen it) gives a row of zeros: nothing outside the table is read.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
-                             float* __restrict__ out, int D) {
+                             float* __restrict__ out, int D, int vocab) {
   const int r = blockIdx.x;
   const long long tok = tokens[r];
-  const T* src = table + tok * (long long)D;
+  const bool known = tok >= 0 && tok < vocab;
+  const T* src = table + (known ? tok : 0) * (long long)D;
   float* dst = out + (long long)r * D;
-  for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = to_f32(src[j]);
+  for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = known ? to_f32(src[j]) : 0.0f;
 }
 
 extern "C" int lq_embed(const void* table, int table_dtype, const int* tokens, float* out, int rows,
-                        int D, hipStream_t stream) {
-  LQ_REQUIRE(rows > 0 && D > 0, "embed: rows %d and width %d must be positive", rows, D);
+                        int D, int vocab, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && D > 0 && vocab > 0, "embed: rows %d, width %d and table rows %d must be positive", rows, D, vocab);
   const int threads = D >= 1024 ? 256 : 64;
   if (table_dtype == LQ_F32)
-    embed_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, tokens, out, D);
+    embed_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, tokens, out, D, vocab);
   else if (table_dtype == LQ_BF16)
-    embed_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, tokens, out, D);
+    embed_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab);
   else
     LQ_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
   LQ_CHECK_LAUNCH("embed");

@@ -47,6 +47,38 @@ class GenerationResult:
     batches: int = 0
 
 
+class _Launched:
+    """A decoding step that has been queued: its sequences, and its sampled tokens once they are asked
+    for.  On the GPU the tokens are copied to pinned host memory behind the step, with an event after the
+    copy, so that reading them waits for this step only and not for what was queued after it."""
+
+    def __init__(self, slots: List[int], device_tokens: torch.Tensor, host: Optional[torch.Tensor]) -> None:
+        self.slots = slots
+        n = len(slots)
+        if host is None:
+            self.host = device_tokens[:n].clone()
+            self.event = None
+        else:
+            self.host = host[:n]
+            self.host.copy_(device_tokens[:n], non_blocking=True)
+            self.event = torch.cuda.Event()
+            self.event.record()
+
+    def wait(self) -> None:
+        if self.event is not None:
+            self.event.synchronize()
+            self.event = None
+
+    def tokens(self, slots: List[int]) -> List[int]:
+        """The tokens of `slots`, all or some of the step's sequences, in that order."""
+        self.wait()
+        got = self.host.tolist()
+        if slots == self.slots:
+            return got
+        at = {s: i for i, s in enumerate(self.slots)}
+        return [got[at[s]] for s in slots]
+
+
 class GenerationLoop:
     """Which requests run together, when a sequence ends, what is returned."""
 
@@ -138,6 +170,10 @@ class GenerationLoop:
                     changed = first or survivors != live
                     first = False
                     live = survivors
+                    # whether a step can follow this one, whatever it samples (a backend may run ahead then)
+                    expect = getattr(be, "expect_more", None)
+                    if expect is not None:
+                        expect(any(len(result.tokens[r]) + 1 < limit[r] for r in live))
                     sampled = be.decode([slots[r] for r in live],
                                         [result.tokens[r][-1] for r in live], changed)
                     result.decode_steps += 1
@@ -172,6 +208,15 @@ class EngineBackend:
         self.keep_logits = False
         self.last_logits: Optional[torch.Tensor] = None
         self.prefill_steps = 0
+        # Running ahead: a replayed step takes its tokens from where the step before left them, on the
+        # device, so the step after the one that the loop is asking for can be queued before the host has
+        # seen any token: the device then never waits for the host between steps.  `ahead` is that step
+        # (launched, not yet read); `more` is what the loop said about a step following (`expect_more`).
+        self.run_ahead = True
+        self.ahead: Optional[_Launched] = None
+        self.more = True
+        self.steps_ahead = 0  # steps that were queued before their turn (for tests and curiosity)
+        self._token_buffers: List[torch.Tensor] = []
 
     # ---- what the loop asks ------------------------------------------------------------
     def free_blocks(self) -> int:
@@ -186,7 +231,12 @@ class EngineBackend:
         limit = self.engine.max_sequence_tokens
         return None if limit is None else limit - prompt_tokens + 1
 
+    def expect_more(self, more: bool) -> None:
+        """The loop's word on whether a step can follow the next `decode`, whatever it samples."""
+        self.more = bool(more)
+
     def new_sequence(self, request_index: int, prompt: Sequence[int]) -> int:
+        self._drop_ahead()
         slot = self.engine.new_sequence()
         self.engine.sampler_state.start(slot, sequence_key(self.params.seed, request_index), prompt)
         self.request_of[slot] = request_index
@@ -202,6 +252,7 @@ class EngineBackend:
         tokens of as many sequences as fit, a long prompt goes on in the next step), and samples each
         sequence's first token from the logits at its last place."""
         e = self.engine
+        self._drop_ahead()
         self.current = None
         rows_out: List[Optional[torch.Tensor]] = [None] * len(slots)
         at = [0] * len(slots)  # tokens of each prompt that have run
@@ -233,7 +284,11 @@ class EngineBackend:
         if not self.use_graphs:
             logits = e.step([StepEntry(s, [t], [0]) for s, t in zip(slots, last_tokens)])
             return self._sample_eager(logits, slots)
-        return e.run_on_stream(lambda: self._decode_graph(list(slots), list(last_tokens), changed))
+        # A replayed step follows the prompt step or the step before it on the engine's stream, and the host
+        # waits for its tokens before it does anything else with the sequences: no waits between streams.
+        # (What is queued ahead is waited for in `_drop_ahead` before other work may touch its slots.)
+        step = e.run_on_stream(lambda: self._decode_graph(list(slots), list(last_tokens), changed), handshake=False)
+        return self._checked(step.tokens(list(slots)), slots)
 
     # ---- internals ------------------------------------------------------------------------
     def _checked(self, tokens: List[int], slots: Sequence[int]) -> List[int]:
@@ -257,32 +312,88 @@ class EngineBackend:
 
         return self._checked(e.run_on_stream(body), slots)
 
-    def _decode_graph(self, slots: List[int], last_tokens: List[int], changed: bool) -> List[int]:
+    def _decode_graph(self, slots: List[int], last_tokens: List[int], changed: bool) -> "_Launched":
+        """The launched step whose tokens answer this call: the one queued ahead if it is the step asked
+        for (the same sequences, or some of them: a step's results do not depend on who else was in it),
+        else a step launched now.  Queues the step after it while the device still works on this one."""
+        step, self.ahead = self.ahead, None
+        if step is not None and not (set(slots) <= set(step.slots)):
+            step.wait()  # not what is asked for (the loop never does this): its tokens are dropped
+            step = None
+        if step is None:
+            step = self._launch(slots, last_tokens, changed)
+        elif step.slots != slots:
+            self.current = None  # the batch shrank: its next step starts from arrays written anew
+        if self.run_ahead and self.more and not self.keep_logits and step.slots == slots:
+            self.ahead = self._launch_next(step)
+        return step
+
+    def _launch(self, slots: List[int], last_tokens: Optional[List[int]], changed: bool,
+                same_graph=None) -> Optional["_Launched"]:
+        """Queues one decoding step.  With `same_graph` (running ahead) only if that very graph takes the
+        step as its arrays stand: None otherwise, and nothing has changed."""
         e = self.engine
         cache = e.cache
         starts = [cache.length(s) for s in slots]
-        for s, n in zip(slots, starts):
-            e.check_room(s, n, 1)
-        growth = {s: 1 for s in slots}
-        cache.reserve(growth)
         longest = max(starts) + 1
         bound = (longest + LEN_BUCKET - 1) // LEN_BUCKET * LEN_BUCKET
-        g, fresh = self.graphs.get(len(slots), bound)
-        # a graph's arrays carry on from its own last step only: anything else in between (another graph,
-        # a prompt step, a batch whose members changed) means they are written anew
-        if fresh or changed or g is not self.current or g.slots != slots:
-            g.load(slots, last_tokens, starts)
-        if fresh:
-            g.capture(self.sampler)
+        growth = {s: 1 for s in slots}
+        if same_graph is not None:
+            if bound != same_graph.bound:
+                return None
+            try:
+                for s, n in zip(slots, starts):
+                    e.check_room(s, n, 1)
+                cache.reserve(growth)
+            except (SequenceTooLong, CacheFull):
+                return None  # the loop meets the same error when (and if) it asks for this step
+            g = same_graph
+        else:
+            for s, n in zip(slots, starts):
+                e.check_room(s, n, 1)
+            cache.reserve(growth)
+            g, fresh = self.graphs.get(len(slots), bound)
+            # a graph's arrays carry on from its own last step only: anything else in between (another graph,
+            # a prompt step, a batch whose members changed) means they are written anew
+            if fresh or changed or g is not self.current or g.slots != slots:
+                g.load(slots, last_tokens, starts)
+            if fresh:
+                g.capture(self.sampler)
         self.current = g
         g.launch()
         cache.advance(growth)
         e.steps_run += 1
         if self.keep_logits:
             self.last_logits = g.logits.clone()
-        return self._checked(g.views[0].cpu().tolist(), slots)
+        return _Launched(list(slots), g.views[0], self._token_buffer(len(slots)))
+
+    def _launch_next(self, step: "_Launched") -> Optional["_Launched"]:
+        nxt = self._launch(step.slots, None, False, same_graph=self.current)
+        if nxt is not None:
+            self.steps_ahead += 1
+        return nxt
+
+    def _token_buffer(self, n: int) -> Optional[torch.Tensor]:
+        """Pinned host memory for a step's tokens; two buffers take turns (the step ahead and the one
+        before it).  None off the GPU, where a copy is taken at once."""
+        if self.engine.device.type != "cuda":
+            return None
+        if not self._token_buffers or self._token_buffers[0].numel() < n:
+            self._token_buffers = [torch.empty(max(n, 64), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._token_buffers.reverse()
+        return self._token_buffers[0]
+
+    def _drop_ahead(self) -> None:
+        """A step queued ahead that nobody will ask for (its batch ended, or other work comes first): it has
+        run or will run before anything queued after it, and what it wrote belongs to slots that are
+        given back or written anew."""
+        if self.ahead is not None:
+            self.ahead.wait()
+            self.ahead = None
+            self.current = None
 
     def close(self) -> None:
+        self._drop_ahead()
         if self.graphs is not None:
             self.graphs.close()
         self.current = None

@@ -114,7 +114,7 @@ class HipKernels:
 
     # ------------------------------------------------------------------ kernels
     def embed(self, table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
-        """out[r, :] = float32(table[tokens[r], :])"""
+        """out[r, :] = float32(table[tokens[r], :]); zeros where tokens[r] is no row of the table"""
         self._dev(table, tokens, out)
         rows, width = out.shape
         self._i32(tokens, "embed tokens", rows)
@@ -123,7 +123,7 @@ class HipKernels:
         if table.dim() != 2 or table.shape[1] != width:
             raise KernelLibraryError(f"embed: table {tuple(table.shape)} does not match width {width}")
         self._check(self.lib.lq_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(out),
-                                      c_int(rows), c_int(width), self.stream))
+                                      c_int(rows), c_int(width), c_int(table.shape[0]), self.stream))
 
     @staticmethod
     def _pieces(delta: Optional[torch.Tensor], like: torch.Tensor, what: str):

@@ -26,7 +26,9 @@ class CpuKernels:
         pass
 
     def embed(self, table, tokens, out):
-        out.copy_(table[tokens[: out.shape[0]].long()].float())
+        t = tokens[: out.shape[0]].long()
+        known = (t >= 0) & (t < table.shape[0])  # no row of the table: zeros, as the library does
+        out.copy_(table[t.clamp(0, table.shape[0] - 1)].float() * known[:, None])
 
     @staticmethod
     def _whole(delta, like):

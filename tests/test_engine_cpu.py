@@ -225,6 +225,38 @@ def test_a_batch_after_another_of_the_same_size_loads_its_graph_anew(tmp_path, n
     assert eng.cache.slots.taken_count == 0
 
 
+def test_steps_queued_ahead_give_the_same_tokens_and_none_is_wasted_at_a_known_end(tmp_path):
+    """A replayed step takes its tokens from where the last one left them, so the backend queues the next
+    step before the host has read this one's tokens.  The tokens are those of direct steps, also when a
+    sequence ends on a stop id in the middle (the step queued ahead then ran for a batch with one sequence
+    too many: the others' tokens are taken from it) and when a batch ends and another follows on the same
+    slots.  Where every sequence ends by its limit the loop says so, and no step is queued in vain."""
+    from longbow_quarrel_amd.engine.generate import EngineBackend, GenerationLoop
+
+    eng, ref = make(tmp_path, TINY_A)
+    prompts = [random_tokens(3 + 2 * i, 256, 70 + i) for i in range(5)]
+    direct = lq.generate(eng, prompts, 6, stop_ids=[], use_graphs=False)
+    stop = direct.tokens[1][2]  # request 1 ends on its third token; whoever else samples it ends there too
+    expect = lq.generate(eng, prompts, 6, stop_ids=[stop], use_graphs=False)
+    assert expect.finish[1] == "stop" and "length" in expect.finish
+    graphs_cls, log = _replayed_graphs()
+    for ahead in (True, False):
+        del log[:]
+        be = EngineBackend(eng, lq.SamplingParams(), graphs_cls=graphs_cls)
+        be.run_ahead = ahead
+        res = GenerationLoop(be, max_batch=3).run(prompts, 6, stop_ids=[stop])
+        assert res.tokens == expect.tokens and res.finish == expect.finish, ahead
+        assert (be.steps_ahead > 0) == ahead
+        launches = sum(1 for e in log if e[0] == "launch")
+        assert launches >= res.decode_steps and (ahead or launches == res.decode_steps)
+        del log[:]
+        res = GenerationLoop(be, max_batch=3).run(prompts, 6, stop_ids=[])
+        assert res.tokens == direct.tokens
+        assert sum(1 for e in log if e[0] == "launch") == res.decode_steps  # every sequence ends by its limit
+        be.close()
+        assert be.ahead is None and eng.cache.slots.taken_count == 0
+
+
 def test_prompts_run_in_portions_of_at_most_max_prefill_rows(tmp_path):
     """A batch's prompts are fed in steps of a bounded number of rows: several sequences a step, a long
     prompt over several steps (cut at 2 tokens, at a cache block's edge, anywhere), logits only from each

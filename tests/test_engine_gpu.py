@@ -193,6 +193,29 @@ def test_generation_in_bfloat16_graphs_and_direct_steps_agree(tmp_path_factory):
     assert alone.tokens[0] == batch.tokens[0]
 
 
+def test_steps_queued_ahead_of_the_host_and_a_sequence_that_stops_in_between(tmp_path_factory):
+    """Captured steps are queued one ahead of the host.  A sequence that ends on a stop id leaves a step
+    behind that ran for one sequence too many; the others go on from that step's tokens.  Greedy and seeded
+    sampling through graphs equal direct steps, with run-ahead and without it."""
+    from longbow_quarrel_amd.engine.generate import EngineBackend, GenerationLoop
+
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, "c_sharp", "bfloat16")
+    prompts = [reqs[1], reqs[2], reqs[4], reqs[0]]
+    for params in (lq.SamplingParams(), lq.SamplingParams(temperature=0.9, top_k=50, seed=11)):
+        free = lq.generate(eng, prompts, 24, params, stop_ids=[], use_graphs=False)
+        stop = free.tokens[2][7]
+        direct = lq.generate(eng, prompts, 24, params, stop_ids=[stop], use_graphs=False)
+        assert direct.finish[2] == "stop" and "length" in direct.finish
+        for ahead in (True, False):
+            be = EngineBackend(eng, params)
+            be.run_ahead = ahead
+            got = GenerationLoop(be, max_batch=3).run(prompts, 24, stop_ids=[stop])
+            assert got.tokens == direct.tokens and got.finish == direct.finish, (params, ahead)
+            assert (be.steps_ahead > 0) == ahead
+            be.close()
+    assert eng.cache.slots.taken_count == 0
+
+
 @pytest.mark.parametrize("n_prompts,max_batch", [(6, 3), (2, 1)])
 def test_batches_of_one_size_one_after_another_through_captured_graphs(tmp_path_factory, n_prompts, max_batch):
     """The second batch finds a captured graph of its own size, on the same slots, whose arrays still hold

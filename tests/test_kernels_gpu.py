@@ -39,6 +39,11 @@ def test_embed(kn, dtype, width):
     out = torch.empty((5, width), dtype=torch.float32, device=DEV)
     kn.embed(table, toks, out)
     assert torch.equal(out, table[toks.long()].float())
+    # an id that is no row of the table (the sampler's "no token", an id past the end) gives zeros
+    toks = i32([5, -1, 97, 96, 1 << 30])
+    out.fill_(7.0)
+    kn.embed(table, toks, out)
+    assert torch.equal(out[[0, 3]], table[[5, 96]].float()) and not out[[1, 2, 4]].any()
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
