@@ -574,7 +574,9 @@ def test_toy_parts_on_the_gpu(dtype):
         tensors = {k: v.cpu() for k, v in random_tensors(eng.model.tensor_specs(), 3, eng.dtype, 0.2, device=eng.device).items()}
         a, b = random_tokens(40, 53, 1), random_tokens(9, 53, 2)
         wa, wb = (toy_parts.plain_toy(toy_parts.TOY, tensors, t) for t in (a, b))
-        limit = TOL_F32 if dtype == "float32" else 6e-2  # no rounding hooks in the toy's plain twin
+        # the toy's plain twin rounds nothing: with weights of standard deviation 0.2 the engine's bfloat16
+        # activations differ from it by 0.7e-2 to 1.9e-2 over several seeds; the 32-bit run is what pins the parts
+        limit = TOL_F32 if dtype == "float32" else 3e-2
         sa, sb = eng.new_sequence(), eng.new_sequence()
         out = eng.step([StepEntry(sa, a[:17], range(17)), StepEntry(sb, b[:8], range(8))])
         assert rel_err(out[:17], wa[:17]) < limit and rel_err(out[17:], wb[:8]) < limit
