@@ -18,7 +18,10 @@ methods, so that the decisions can be tested without a GPU; `EngineBackend` is t
 real one.  It feeds a batch's prompts in portions of at most `max_prefill_rows` rows
 (the step's workspace grows with its rows, not with the batch), and it reports a row of
 logits that holds a NaN or an infinity as `NonFiniteLogits` where the reference takes
-the first finite index (internal/engine/sampler.go:72-75, 107-123).
+the first finite index (internal/engine/sampler.go:72-75, 107-123).  Replayed decoding steps
+are queued one ahead of the host (`_Launched`, `EngineBackend.ahead`): the device goes from one
+step to the next without waiting for the loop's decisions, which arrive a step late and are
+applied to the step that is already there.
 """
 from __future__ import annotations
 
