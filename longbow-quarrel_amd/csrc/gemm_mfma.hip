@@ -996,8 +996,21 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
     const double c256 = 0.95 * lq_ceil_div(tm * lq_ceil_div(N, 256), cus);
     const double c224 = 1.13 * lq_ceil_div(tm * lq_ceil_div(N, 224), cus);
     const double c192 = 0.78 * lq_ceil_div(tm * lq_ceil_div(N, 192), cus);
-    if (c256 <= c224 && c256 <= c192)
+    if (c256 <= c224 && c256 <= c192) {
+      // Whole rounds of 256-column tiles, and where what is left would fill half a round or less, that rest
+      // as 128-column tiles in a launch of its own: a round of half-size tiles instead of a round of whole
+      // tiles on half the chip (2 048 x 28 672: three rounds and 256 half tiles instead of 3.5 rounds).
+      const int tn = lq_ceil_div(N, 256), rest = (tm * tn) % cus;
+      if (N % 256 == 0 && tm * tn > cus && 4 * rest >= cus && rest % tm == 0 && 2 * rest <= cus + cus / 8) {
+        const int n1 = (tn - rest / tm) * 256, n2 = N - n1;
+        const int col2 = EPI == EPI_SWIGLU ? n1 / 2 : n1;  // where the second launch's columns start in out
+        int rc = launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, n1, K, lda, ldw, ldc, 1, 0, stream);
+        if (rc != 0) return rc;
+        return launch_pipelined<4, 2, 2, 2, 64, 2, EPI, TO, true>(x, (const bf16_t*)w + (long long)n1 * ldw,
+                                                                  (TO*)out + col2, M, n2, K, lda, ldw, ldc, 1, 0, stream);
+      }
       return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    }
     if (c224 <= c192)
       return launch_pipelined<8, 1, 1, 7, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     return launch_pipelined<4, 2, 2, 3, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);

@@ -123,6 +123,9 @@ def test_linear_float32(kn, m, n, k):
     (50, 12800, 512), (100, 12800, 512), (200, 12800, 512),                                # their 64-column siblings
     (1000, 12700, 192), (300, 49000, 64), (2048, 6144, 4096),     # pipelined, 256 x 256 tiles
     (1000, 8200, 96), (130, 66000, 32), (2048, 4096, 4000),        # pipelined, 128 x 256 tiles
+    (2400, 6144, 128), (3100, 7168, 64),   # more than 8 row tiles: an XCD walks windows of 8 x 4 tiles
+    (2048, 28672, 128),                    # 3.5 rounds of tiles: the last half round as 128-column tiles
+    (2048, 6144, 192), (300, 6200, 128),   # 256 x 192 tiles, with an edge
 ])
 def test_linear_bfloat16_matrix_cores(kn, out_dtype, m, n, k):
     x, w = rnd((m, k), 12, torch.bfloat16), rnd((n, k), 13, torch.bfloat16)
@@ -447,6 +450,8 @@ def test_linear_with_fused_swiglu(kn, m, inner, k):
     (every kernel of the product has this epilogue: the GEMVs, the tiled and the pipelined ones)."""
     if inner == 14336 and m == 65:
         m = 130
+    if inner == 1032 and m == 400:
+        m, inner, k = 2048, 14336, 128  # 3.5 rounds of 256 x 256 tiles: the last half round goes as 128-column tiles
     x = rnd((m, k), 41, torch.bfloat16)
     gate, up = rnd((inner, k), 42, torch.bfloat16, 0.05), rnd((inner, k), 43, torch.bfloat16, 0.05)
     assert kn.linear_swiglu_supported(torch.bfloat16, 2 * inner, k)
