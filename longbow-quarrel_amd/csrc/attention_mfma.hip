@@ -519,6 +519,231 @@ int launch_rows(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
   return 0;
 }
 
+// ------------------------------------------------------------------ rows, 32 x 32 score tiles
+// The same launch shape with the wider product, v_mfma_f32_32x32x16_bf16: a wave owns 32 consecutive
+// rows of one query head, a block is the HW query heads of one kv head over the same 32 rows.  A K or
+// V^T fragment read from LDS (1 KB) now feeds a product of 32 x 32 x 16 instead of 16 x 16 x 32: half
+// the LDS traffic a flop, which is what bounded the narrower tile.
+//   lane l gives A[row l%32][k (l/32)*8 .. +8] and B[col l%32][the same k]; it receives
+//   D[(e/4)*8 + (l/32)*4 + e%4][l%32], e < 16.
+//   First product: A = 32 keys x 16 of head_dim (LDS), B = 32 rows x the same 16 (registers):
+//   S^T[key][row]; lane (row r, half h) holds keys (e/4)*8 + 4 h + e%4 of the chunk.
+//   Second product, two steps of 16 keys: step s takes the lane's probabilities e = 8 s .. 8 s + 7 as
+//   they are, so its k index 8 h + j stands for key 16 s + (j/4)*8 + 4 h + j%4; V^T lies in LDS with
+//   the keys of every 16 in the order [0-3][8-11][4-7][12-15], which makes those eight one 16-byte run.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int HD, int HW>
+__global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int heads_per_block_group, int tiles,
+                                                                 int units) {
+  using L = RowsLds<HD>;
+  constexpr int ROWS = 32, THREADS = HW * 64;
+  constexpr int PER_THREAD = (L::PIECES + THREADS - 1) / THREADS;  // pieces of K, and of V, per thread
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  // tasks as in attn_rows_kernel: late (heavy) tiles first, dealt out over the compute units in a snake
+  const int per_tile = gridDim.x / tiles;
+  const int round = blockIdx.x / units, place = blockIdx.x % units;
+  int task = round * units + ((round & 1) ? units - 1 - place : place);
+  if ((round + 1) * units > (int)gridDim.x) task = blockIdx.x;
+  const int head_group = task % per_tile;
+  int t = tiles - 1 - task / per_tile, b = 0, r0 = -1, nrows = 0;
+  for (; b < a.batch; ++b) {
+    const int begin = a.cu_rows[b], n = a.cu_rows[b + 1] - begin;
+    const int tiles_b = (n + ROWS - 1) / ROWS;
+    if (t < tiles_b) {
+      r0 = begin + t * ROWS;
+      nrows = min(ROWS, n - t * ROWS);
+      break;
+    }
+    t -= tiles_b;
+  }
+  if (r0 < 0) return;  // the whole block
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c32 = lane & 31, hf = lane >> 5;
+  const int G = a.nh / a.nkv;
+  const int kvh = head_group / heads_per_block_group;
+  const int hq = (head_group % heads_per_block_group) * HW + wave;
+  const bool wave_active = hq < G;  // an idle wave still copies and meets the barriers
+  const int h = kvh * G + min(hq, G - 1);
+  const int* table = a.block_table + (long long)a.seq_slot[b] * a.bt_stride;
+  const int p0 = a.row_pos[r0];
+
+  // this lane's row (column of the score tile)
+  const int rc = min(c32, nrows - 1);
+  const bool valid = wave_active && c32 < nrows;
+  const int pos = p0 + rc;
+  const int lo = (a.window > 0 && pos >= a.window) ? pos - a.window + 1 : 0;
+  const int last_key = wave_active ? p0 + nrows - 1 : -1;                       // wave-uniform
+  const int first_key = (a.window > 0 && p0 >= a.window) ? p0 - a.window + 1 : 0;
+  // keys up to the first row's position and from the last row's window start on are visible to all 32 rows
+  const int free_to = (wave_active && nrows == ROWS) ? p0 : -1;
+  const int free_from = (a.window > 0 && p0 + nrows - 1 >= a.window) ? p0 + nrows - 1 - a.window + 1 : 0;
+  bf16x8 q[HD / 16];
+  {
+    const bf16_t* qr = a.q + (long long)(r0 + rc) * a.ldq + h * HD + hf * 8;
+#pragma unroll
+    for (int kk = 0; kk < HD / 16; ++kk) q[kk] = as_bf16x8(*(const u32x4*)(qr + kk * 16));
+  }
+  f32x16 o[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[dt][e] = 0.f;
+  float m = -INFINITY, l = 0.f;  // running maximum of the row (log2 domain); this lane's share of the normaliser
+
+  const int t_end = p0 + nrows - 1;  // the last key anyone here sees, and the last one written
+  const int blk_first = first_key / BS, blk_last = t_end / BS;
+
+  u32x4 rk[PER_THREAD], rv[PER_THREAD];
+  auto fetch = [&](int lb) {
+    const long long blk = table[lb];
+    const bf16_t* kb = a.kcache + (blk * a.nkv + kvh) * (long long)(BS * HD);
+    const bf16_t* vb = a.vcache + (blk * a.nkv + kvh) * (long long)(HD * BS);
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int pc = tid + i * THREADS;
+      if (pc < L::PIECES) {
+        rk[i] = *(const u32x4*)(kb + pc * 8);
+        rv[i] = *(const u32x4*)(vb + pc * 8);
+      }
+    }
+  };
+  auto stash = [&](int lb, unsigned char* stage) {
+    // values of keys that were never written must not reach the product (0 * garbage may be NaN)
+    const int base_key = lb * BS;
+    const bool tail = base_key + BS - 1 > t_end;
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const int pc = tid + i * THREADS;
+      if (pc < L::PIECES) {
+        const int key = pc / (HD / 8), part = pc % (HD / 8);  // keys in their own order: row = key
+        *(u32x4*)(stage + key * L::K_STRIDE + part * 16) = rk[i];
+        const int d = pc >> 3, vpart = pc & 7;  // eight keys of one d: 8 vpart .. + 7
+        u32x4 v = rv[i];
+        if (tail) {
+          const int k0 = base_key + vpart * 8;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (k0 + 2 * e > t_end) v[e] &= 0xffff0000u;
+            if (k0 + 2 * e + 1 > t_end) v[e] &= 0x0000ffffu;
+          }
+        }
+        // within every 16 keys the order in LDS is [0-3][8-11][4-7][12-15]
+        unsigned char* vrow = stage + L::K_BYTES + d * L::V_STRIDE + (vpart >> 1) * 32;
+        const int odd = vpart & 1;
+        *(u32x2*)(vrow + (odd ? 8 : 0)) = (u32x2){v[0], v[1]};
+        *(u32x2*)(vrow + (odd ? 24 : 16)) = (u32x2){v[2], v[3]};
+      }
+    }
+  };
+
+  fetch(blk_first);
+  stash(blk_first, smem);
+  __syncthreads();
+  for (int lb = blk_first; lb <= blk_last; ++lb) {
+    unsigned char* cur = smem + ((lb - blk_first) & 1) * L::STAGE;
+    unsigned char* nxt = smem + ((lb - blk_first + 1) & 1) * L::STAGE;
+    const bool more = lb < blk_last;
+    if (more) fetch(lb + 1);  // on their way during this block's products
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int t0 = lb * BS + half * 32;
+      if (t0 > t_end) break;
+      if (t0 > last_key || t0 + 31 < first_key) continue;  // nothing of this chunk is visible to this wave
+      f32x16 sc;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sc[e] = 0.f;
+      const unsigned char* kr = cur + (half * 32 + c32) * L::K_STRIDE + hf * 16;
+#pragma unroll
+      for (int kk = 0; kk < HD / 16; ++kk)
+        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(*(const u32x4*)(kr + kk * 32)), q[kk], sc, 0, 0, 0);
+      const bool masked = !(t0 + 31 <= free_to && t0 >= free_from);
+      if (masked) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int tk = t0 + (e >> 2) * 8 + hf * 4 + (e & 3);
+          if (!(valid && tk >= lo && tk <= pos)) sc[e] = -INFINITY;
+        }
+      }
+      float cmax = sc[0];
+#pragma unroll
+      for (int e = 1; e < 16; ++e) cmax = fmaxf(cmax, sc[e]);
+      {  // the row's other sixteen keys are in the lane 32 places away
+        auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(cmax), __float_as_uint(cmax), false, false);
+        cmax = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+      }
+      const float m_new = fmaxf(m, cmax * a.scale_log2);  // the scale is positive: it commutes with the maximum
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row with no key yet
+      const float alpha = fast_exp2(m - m_safe);
+      float psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        sc[e] = fast_exp2(fmaf(sc[e], a.scale_log2, -m_safe));  // -inf stays -inf, 2^-inf = 0
+        psum += sc[e];
+      }
+      l = l * alpha + psum;
+      m = m_new;
+      u32x4 pw[2];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pw[s2][j] = pack_bf16(sc[8 * s2 + 2 * j], sc[8 * s2 + 2 * j + 1]);
+      if (!__all(alpha == 1.0f)) {  // the maximum moved for some row: rescale what has been summed
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+      }
+      const unsigned char* vr = cur + L::K_BYTES + c32 * L::V_STRIDE + half * 64 + hf * 16;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(*(const u32x4*)(vr + dt * 32 * L::V_STRIDE + s2 * 32)),
+                                                          as_bf16x8(pw[s2]), o[dt], 0, 0, 0);
+    }
+    // Nobody reads nxt: its last readers passed the barrier below one round ago.
+    if (more) stash(lb + 1, nxt);
+    __syncthreads();
+  }
+  {
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l), __float_as_uint(l), false, false);
+    l = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+  }
+  if (!valid) return;
+  const float inv = 1.0f / l;
+  bf16_t* orow = a.out + (long long)(r0 + c32) * a.ldo + h * HD + hf * 4;
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {  // d = dt*32 + g4*8 + hf*4 + (0..3)
+      u32x2 ww;
+      ww[0] = pack_bf16(o[dt][g4 * 4 + 0] * inv, o[dt][g4 * 4 + 1] * inv);
+      ww[1] = pack_bf16(o[dt][g4 * 4 + 2] * inv, o[dt][g4 * 4 + 3] * inv);
+      *(u32x2*)(orow + dt * 32 + g4 * 8) = ww;
+    }
+}
+
+template <int HD, int HW>
+int launch_rows32(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
+  using L = RowsLds<HD>;
+  const size_t smem = 2 * (size_t)L::STAGE;
+  auto kernel = attn_rows32_kernel<HD, HW>;
+  static bool configured = false;
+  if (!configured && smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      lq_set_error("attention: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+      return -2;
+    }
+    configured = true;
+  }
+  const int tiles = lq_ceil_div(rows, 32) + a.batch;  // an upper bound: a sequence's last tile may be partial
+  kernel<<<dim3(tiles * a.nkv * groups), HW * 64, smem, stream>>>(a, groups, tiles, lq_compute_units());
+  LQ_CHECK_LAUNCH("attention(mfma rows, 32 x 32)");
+  return 0;
+}
+
 // ------------------------------------------------------------------ heads (decoding)
 // Block = NW waves over one split of one (sequence, kv head).  LDS: per wave HD x G floats of
 // partial output (the valid columns only), G maxima, G normalisers.
@@ -731,6 +956,20 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
   if (!decode) {
     constexpr int QT = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
     constexpr int QT2 = QT > 1 ? QT / 2 : 1;  // with two row groups of waves: the same rows a block, half a wave
+    if constexpr (HD % 32 == 0 && HD <= 128) {
+      // The 32 x 32 score tile (its accumulators fit up to this head size) reads half as much from LDS for a
+      // product, with half as many waves on a compute unit to hide one wave's softmax behind another's
+      // products.  As measured (32 heads over 8, one sequence): at head size 64 it wins at every length
+      // (46 against 68 us at 2 048 tokens, 353 against 429 at 8 192), at 96 and 128 from about 3 000 tokens a
+      // sequence on (644 against 682 us at 8 192, 76 against 68 at 2 048); with fewer than four heads a
+      // kv head it wins throughout.
+      const bool wide = HD <= 64 || G < 4 || rows >= 3072 * a.batch;
+      if (wide && G >= 4) return launch_rows32<HD, 4>(a, rows, lq_ceil_div(G, 4), stream);
+      if (wide && G >= 2) return launch_rows32<HD, 2>(a, rows, lq_ceil_div(G, 2), stream);
+      // (one wave a block would have to stage a whole cache block through its own registers)
+      if constexpr (HD <= 64)
+        if (wide && G == 1) return launch_rows32<HD, 1>(a, rows, 1, stream);
+    }
     if (G >= 4) return launch_rows<HD, QT2, 4, 2>(a, rows, lq_ceil_div(G, 4), stream);
     if (G >= 2) return launch_rows<HD, QT, 2, 1>(a, rows, lq_ceil_div(G, 2), stream);
     return launch_rows<HD, QT, 1, 1>(a, rows, 1, stream);

@@ -322,6 +322,21 @@ def test_attention_prompts(kn, dtype, generic, heads, kv_heads, head_dim):
     assert rel_err(got, want) < (2e-6 if dtype == torch.float32 else 8e-3)
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,lengths,new,window", [
+    (8, 2, 64, [5, 70, 131, 1, 300], [5, 70, 40, 1, 300], 0),   # four heads a kv head, head size 64: 32 x 32 tiles
+    (8, 2, 64, [200, 333], [200, 100], 90),                      # and with a window
+    (16, 2, 128, [3100], [3100], 0),                             # head size 128: 32 x 32 tiles from 3 072 rows a sequence
+    (8, 2, 128, [3200], [3200], 1000),
+    (8, 2, 96, [100, 3200 * 2 - 100], [100, 3200 * 2 - 100], 0), # two sequences, 3 200 rows on average
+    (8, 2, 128, [700, 64, 257], [700, 64, 200], 0),              # short sequences of head size 128: 16 x 16 tiles
+])
+def test_attention_prompts_on_both_tile_shapes(kn, heads, kv_heads, head_dim, lengths, new, window):
+    """Prompt attention has a kernel with 32 x 32 score tiles and one with 16 x 16: which one runs depends on
+    the head size, the heads a kv head and the rows a sequence.  Both against the plain implementation."""
+    got, want = run_attention(kn, None, lengths, new, heads, kv_heads, head_dim, torch.bfloat16, 77, window=window)
+    assert rel_err(got, want) < 8e-3
+
+
 @pytest.mark.parametrize("dtype,generic", [(torch.float32, True), (torch.bfloat16, False)])
 @pytest.mark.parametrize("heads,kv_heads,head_dim", [(32, 8, 128), (3, 1, 32), (16, 1, 64), (6, 3, 48)])
 def test_attention_decoding_over_long_keys(kn, dtype, generic, heads, kv_heads, head_dim):
