@@ -2,6 +2,7 @@
 // add folded in), rotation + cache write, SwiGLU, residual add, row gather, casts.
 // Norm statistics, rotation angles and the residual sum are 32-bit (or wider).
 #include "common.h"
+#include <algorithm>
 
 // ---------------------------------------------------------------- embedding
 // out[r, :] = float(table[token[r], :])   (row copy, internal/device/kernels.metal:465-467)
@@ -435,8 +436,12 @@ __device__ inline void rotate8(u32x4_t& a, u32x4_t& b, const float* c, const flo
     const float x0a = __uint_as_float(a[j] << 16), x0b = __uint_as_float(a[j] & 0xffff0000u);
     const float x1a = __uint_as_float(b[j] << 16), x1b = __uint_as_float(b[j] & 0xffff0000u);
     const float ca = c[2 * j], cb = c[2 * j + 1], sa = s[2 * j], sb = s[2 * j + 1];
-    a[j] = (unsigned)f32_to_bf16(x0a * ca - x1a * sa).bits | ((unsigned)f32_to_bf16(x0b * cb - x1b * sb).bits << 16);
-    b[j] = (unsigned)f32_to_bf16(x0a * sa + x1a * ca).bits | ((unsigned)f32_to_bf16(x0b * sb + x1b * cb).bits << 16);
+    // one rounded product and one fused multiply-add, spelt out: left to the compiler, which of the two
+    // products is fused differs from one caller to the next, and so does the last bit where they cancel
+    const float ra = __fmaf_rn(x0a, ca, -__fmul_rn(x1a, sa)), rb = __fmaf_rn(x0b, cb, -__fmul_rn(x1b, sb));
+    const float ia = __fmaf_rn(x0a, sa, __fmul_rn(x1a, ca)), ib = __fmaf_rn(x0b, sb, __fmul_rn(x1b, cb));
+    a[j] = (unsigned)f32_to_bf16(ra).bits | ((unsigned)f32_to_bf16(rb).bits << 16);
+    b[j] = (unsigned)f32_to_bf16(ia).bits | ((unsigned)f32_to_bf16(ib).bits << 16);
   }
 }
 
@@ -498,6 +503,144 @@ __global__ __launch_bounds__(256) void rope_store_vec_kernel(
       dst[(long long)(2 * j + 1) * BS] = hi;
     }
   }
+}
+
+// The same for the rows of prompts, eight positions at a time: a block takes the rows of one sequence whose
+// positions lie in one group [8 g, 8 g + 8), so that the values of a whole group go into the transposed V
+// cache as runs of eight positions (16 bytes) instead of two bytes at a time, and takes cos and sin from
+// the step's table (cs[row][pair][2], the same numbers that the kernels above work out for themselves).
+// Blocks are counted sequence by sequence; a sequence's first and last group may be partial.
+__global__ __launch_bounds__(256) void rope_store_groups_kernel(
+    bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v, int ldq, int ldk, int ldv,
+    int nh, int nkv, int hd, const float* __restrict__ cs, const int* __restrict__ row_pos,
+    const int* __restrict__ cu_rows, int batch, const int* __restrict__ seq_slot,
+    const int* __restrict__ block_table, int bt_stride, bf16_t* __restrict__ kcache, bf16_t* __restrict__ vcache,
+    int BS) {
+  int t = blockIdx.x, b = 0, r_begin = 0, n = 0, start = 0;
+  for (; b < batch; ++b) {
+    r_begin = cu_rows[b];
+    n = cu_rows[b + 1] - r_begin;
+    if (n <= 0) continue;
+    start = row_pos[r_begin];
+    const int groups = (start % 8 + n + 7) / 8;
+    if (t < groups) break;
+    t -= groups;
+  }
+  if (b >= batch) return;  // the whole block: the grid is an upper bound
+  const int g8 = (start / 8 + t) * 8;
+  const int p_lo = max(g8, start), p_hi = min(g8 + 8, start + n);
+  const int r_lo = r_begin + (p_lo - start), cnt = p_hi - p_lo;  // rows r_lo .. r_lo + cnt - 1, positions p_lo ..
+  const long long blk = block_table[(long long)seq_slot[b] * bt_stride + p_lo / BS];
+  const int off0 = p_lo % BS;
+  const int half = hd / 2, hv = half / 8;
+
+  // A rotation item: 8 pairs (i .. i + 7, partners half further) of one head of one row.  Four items' loads
+  // are asked for before the first is rotated: the items of a thread are independent, and their round trips
+  // to memory would otherwise follow one another.
+  struct Item {
+    u32x4_t a, b;
+    float4 t[4];
+  };
+  auto load_item = [&](const bf16_t* src, int row, int h, int i, Item& x) {
+    x.a = *(const u32x4_t*)(src + h * hd + i);
+    x.b = *(const u32x4_t*)(src + h * hd + half + i);
+    const float4* t4 = (const float4*)(cs + ((long long)row * half + i) * 2);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) x.t[j] = t4[j];
+  };
+  auto finish_item = [&](Item& x, bf16_t* dst, int i) {
+    float c[8], sn[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      c[2 * j] = x.t[j].x;
+      sn[2 * j] = x.t[j].y;
+      c[2 * j + 1] = x.t[j].z;
+      sn[2 * j + 1] = x.t[j].w;
+    }
+    rotate8(x.a, x.b, c, sn);
+    *(u32x4_t*)(dst + i) = x.a;
+    *(u32x4_t*)(dst + half + i) = x.b;
+  };
+  // the query heads are shared out over gridDim.y blocks; the last of them also takes the keys and the values
+  const int parts = gridDim.y, part = blockIdx.y;
+  const int h_lo = nh * part / parts, h_n = nh * (part + 1) / parts - h_lo;
+  const int q_items = cnt * h_n * hv;
+  for (int it0 = threadIdx.x; it0 < q_items; it0 += 4 * blockDim.x) {
+    Item x[4];
+    bf16_t* dst[4];
+    int ii[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int it = min(it0 + u * (int)blockDim.x, q_items - 1);  // (a repeated last item is written twice alike)
+      const int j = it / (h_n * hv), rem = it - j * (h_n * hv), h = h_lo + rem / hv;
+      ii[u] = (rem % hv) * 8;
+      bf16_t* qr = q + (long long)(r_lo + j) * ldq;
+      dst[u] = qr + h * hd;
+      load_item(qr, r_lo + j, h, ii[u], x[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (it0 + u * (int)blockDim.x < q_items) finish_item(x[u], dst[u], ii[u]);
+  }
+  if (part != parts - 1) return;
+  const int k_items = cnt * nkv * hv;
+  for (int it0 = threadIdx.x; it0 < k_items; it0 += 2 * blockDim.x) {
+    Item x[2];
+    bf16_t* dst[2];
+    int ii[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int it = min(it0 + u * (int)blockDim.x, k_items - 1);
+      const int j = it / (nkv * hv), rem = it - j * (nkv * hv), h = rem / hv;
+      ii[u] = (rem % hv) * 8;
+      dst[u] = kcache + ((blk * nkv + h) * BS + off0 + j) * (long long)hd;
+      load_item(k + (long long)(r_lo + j) * ldk, r_lo + j, h, ii[u], x[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      if (it0 + u * (int)blockDim.x < k_items) finish_item(x[u], dst[u], ii[u]);
+  }
+  const bf16_t* vr = v + (long long)r_lo * ldv;
+  if (cnt == 8) {  // a whole group: position off0 is a multiple of 8, the run is 16 bytes and aligned
+    for (int c = threadIdx.x; c < nkv * hd; c += blockDim.x) {
+      u32x4_t run;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        run[j] = (unsigned)vr[(long long)(2 * j) * ldv + c].bits | ((unsigned)vr[(long long)(2 * j + 1) * ldv + c].bits << 16);
+      *(u32x4_t*)(vcache + (blk * nkv * hd + c) * (long long)BS + off0) = run;
+    }
+  } else {
+    for (int it = threadIdx.x; it < cnt * nkv * hd; it += blockDim.x) {
+      const int j = it / (nkv * hd), c = it - j * (nkv * hd);
+      vcache[(blk * nkv * hd + c) * (long long)BS + off0 + j] = vr[(long long)j * ldv + c];
+    }
+  }
+}
+
+// q rotated in place, rotated k and v into the cache, for the rows of a step that are laid out sequence by
+// sequence (cu_rows) with consecutive positions: bfloat16, head sizes in steps of 16, aligned rows.
+extern "C" int lq_rope_store_groups(void* q, const void* k, const void* v, int rows, int ldq, int ldk, int ldv,
+                                    int nh, int nkv, int hd, const float* cos_sin, const int* row_pos,
+                                    const int* cu_rows, int batch, const int* seq_slot, const int* block_table,
+                                    int bt_stride, void* kcache, void* vcache, int block_size, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && batch > 0, "rope_store: rows %d and sequences %d must be positive", rows, batch);
+  LQ_REQUIRE(hd > 0 && hd % 16 == 0 && nh > 0 && nkv > 0, "rope_store (groups): head size %d, heads %d / %d", hd, nh, nkv);
+  LQ_REQUIRE(ldq >= nh * hd && ldk >= nkv * hd && ldv >= nkv * hd, "rope_store: a row stride is smaller than its row");
+  LQ_REQUIRE(ldq % 8 == 0 && ldk % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 &&
+                 ((uintptr_t)kcache % 16) == 0 && ((uintptr_t)vcache % 16) == 0 && ((uintptr_t)cos_sin % 16) == 0,
+             "rope_store (groups): rows and caches must be 16-byte aligned");
+  LQ_REQUIRE(block_size > 0 && block_size % 8 == 0 && bt_stride > 0, "rope_store: block size %d, table stride %d",
+             block_size, bt_stride);
+  LQ_REQUIRE(q && k && v && cos_sin && row_pos && cu_rows && seq_slot && block_table && kcache && vcache,
+             "rope_store (groups): null argument");
+  const int blocks = rows / 8 + 2 * batch;  // every sequence has at most two partial groups
+  // few groups (a short step): the query heads of a group are shared out over up to four blocks
+  const int parts = std::max(1, std::min(std::min(4, nh), 2 * lq_compute_units() / blocks));
+  rope_store_groups_kernel<<<dim3(blocks, parts), 256, 0, stream>>>(
+      (bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, ldq, ldk, ldv, nh, nkv, hd, cos_sin, row_pos, cu_rows, batch,
+      seq_slot, block_table, bt_stride, (bf16_t*)kcache, (bf16_t*)vcache, block_size);
+  LQ_CHECK_LAUNCH("rope_store (groups)");
+  return 0;
 }
 
 extern "C" int lq_rope_store(void* q, const void* k, const void* v, int dtype, int rows, int ldq,

@@ -317,11 +317,15 @@ class HipKernels:
                    row_pos: torch.Tensor, row_seq: Optional[torch.Tensor] = None,
                    seq_slot: Optional[torch.Tensor] = None, block_table: Optional[torch.Tensor] = None,
                    kcache: Optional[torch.Tensor] = None, vcache: Optional[torch.Tensor] = None,
-                   block_size: int = 0) -> None:
+                   block_size: int = 0, cos_sin: Optional[torch.Tensor] = None,
+                   cu_rows: Optional[torch.Tensor] = None) -> None:
         """Rotate q (in place) and k by the rows' positions; write rotated k and v into the paged cache.
 
         q [rows, >= heads*head_dim], k and v [rows, >= kv_heads*head_dim] (views into one buffer are
         fine); freqs float64 [head_dim/2] or None for no rotation; without a cache only q is rotated.
+        With the step's table of cos and sin (`rope_table`: float32 [rows, head_dim/2, 2]) and `cu_rows`
+        (the rows lie sequence by sequence, positions consecutive within each) a bfloat16 step that stores
+        takes the kernel that works on eight positions at a time; the results are the same bits.
         """
         self._dev(q, k, v, freqs, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
         rows = q.shape[0]
@@ -349,6 +353,23 @@ class HipKernels:
                     not kcache.is_contiguous() or not vcache.is_contiguous():
                 raise KernelLibraryError("rope_store: cache tensors do not have the paged layout")
             bt_stride = int(block_table.stride(0))
+        if (store and cos_sin is not None and cu_rows is not None and freqs is not None and q.dtype == torch.bfloat16
+                and head_dim % 16 == 0 and block_size % 8 == 0):
+            ldq, ldk, ldv = self._rows2d(q, "q"), self._rows2d(k, "k"), self._rows2d(v, "v")
+            aligned = ldq % 8 == 0 and ldk % 8 == 0 and all(t.data_ptr() % 16 == 0 for t in (q, k, kcache, vcache, cos_sin))
+            if aligned:
+                self._dev(cos_sin, cu_rows)
+                if cos_sin.dtype != torch.float32 or tuple(cos_sin.shape) != (rows, head_dim // 2, 2) \
+                        or not cos_sin.is_contiguous():
+                    raise KernelLibraryError("rope_store: cos_sin must be dense float32 [rows, head_dim/2, 2]")
+                if cu_rows.dtype != torch.int32 or cu_rows.numel() < 2:
+                    raise KernelLibraryError("rope_store: cu_rows must be int32 with an entry past the last sequence")
+                self._check(self.lib.lq_rope_store_groups(
+                    _ptr(q), _ptr(k), _ptr(v), c_int(rows), c_int(ldq), c_int(ldk), c_int(ldv), c_int(heads),
+                    c_int(kv_heads), c_int(head_dim), _ptr(cos_sin), _ptr(row_pos), _ptr(cu_rows),
+                    c_int(cu_rows.numel() - 1), _ptr(seq_slot), _ptr(block_table), c_int(bt_stride), _ptr(kcache),
+                    _ptr(vcache), c_int(block_size), self.stream))
+                return
         self._check(self.lib.lq_rope_store(
             _ptr(q), _ptr(k), _ptr(v), c_int(_code(q)), c_int(rows),
             c_int(self._rows2d(q, "q")), c_int(self._rows2d(k, "k") if k is not None else 0),

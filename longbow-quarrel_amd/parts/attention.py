@@ -98,8 +98,11 @@ class GQAttention(Mixer):
             if freqs is None:
                 self.position.apply(q, k, ctx)
             if cache.write:
+                # the step's table of cos and sin, where the position encoding keeps one (the same for every layer)
+                table = self.position.cos_sin(ctx) if freqs is not None and hasattr(self.position, "cos_sin") else None
                 kn.rope_store(q, k, v, self.heads, self.kv_heads, self.head_dim, freqs, ctx.row_pos,
-                              ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size)
+                              ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size,
+                              cos_sin=table, cu_rows=ctx.cu_rows if table is not None else None)
             elif freqs is not None:
                 kn.rope_store(q, None, None, self.heads, 0, self.head_dim, freqs, ctx.row_pos)
             kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,

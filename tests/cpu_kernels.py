@@ -82,8 +82,13 @@ class CpuKernels:
         a, b = v[..., :half].float(), v[..., half:].float()
         return torch.cat([a * c - b * s, a * s + b * c], dim=-1).reshape(rows, heads * hd)
 
+    def rope_table(self, freqs, row_pos, table):
+        ang = row_pos[: table.shape[0]].double()[:, None] * freqs.double()[None, :]
+        table[:, :, 0] = torch.cos(ang).float()
+        table[:, :, 1] = torch.sin(ang).float()
+
     def rope_store(self, q, k, v, heads, kv_heads, head_dim, freqs, row_pos, row_seq=None, seq_slot=None,
-                   block_table=None, kcache=None, vcache=None, block_size=0):
+                   block_table=None, kcache=None, vcache=None, block_size=0, cos_sin=None, cu_rows=None):
         rows = q.shape[0]
         if freqs is not None:
             q[:, : heads * head_dim] = self._rotate(q, heads, head_dim, freqs, row_pos).to(q.dtype)

@@ -458,6 +458,51 @@ def test_rope_store_rotates_and_writes_the_right_rows(kn, dtype):
         < (1e-4 if dtype == torch.float32 else 0.2)
 
 
+@pytest.mark.parametrize("heads,kv_heads,hd", [(32, 8, 128), (6, 3, 48), (8, 2, 64)])
+def test_rope_store_by_groups_of_eight_positions_writes_the_same_bits(kn, heads, kv_heads, hd):
+    """The kernel for prompt rows (eight positions of a sequence a block, cos and sin from the step's table,
+    V into the transposed cache in runs of eight positions) against the kernel that takes a row at a time:
+    sequences that start at any position (a prompt's later portion), of any length, side by side in one step;
+    q, the K cache and the V cache come out bit for bit the same, and nothing else in the caches is touched."""
+    freqs = plain.rope_frequencies(hd, 500000.0).to(DEV)
+    starts, lens = [0, 3, 64, 70, 5, 127, 8], [200, 1, 9, 130, 3, 2, 16]
+    slots = [4, 2, 7, 1, 5, 3, 6]
+    n_blocks, per_seq = 40, 4
+    g = torch.Generator().manual_seed(9)
+    table = torch.randperm(n_blocks, generator=g)[: 8 * per_seq].view(8, per_seq).to(torch.int32).to(DEV)
+    pos, row_seq, cu = [], [], [0]
+    for b, (st, n) in enumerate(zip(starts, lens)):
+        pos += list(range(st, st + n))
+        row_seq += [b] * n
+        cu.append(cu[-1] + n)
+    rows = len(pos)
+    width = (heads + 2 * kv_heads) * hd
+    qkv0 = rnd((rows, width), 33, torch.bfloat16)
+    results = []
+    for grouped in (False, True):
+        qkv = qkv0.clone()
+        kc = torch.full((n_blocks, kv_heads, BS, hd), 3.0, dtype=torch.bfloat16, device=DEV)
+        vc = torch.full((n_blocks, kv_heads, hd, BS), 3.0, dtype=torch.bfloat16, device=DEV)
+        q, k = qkv[:, : heads * hd], qkv[:, heads * hd : (heads + kv_heads) * hd]
+        v = qkv[:, (heads + kv_heads) * hd :]
+        extra = {}
+        if grouped:
+            cs = torch.empty((rows, hd // 2, 2), dtype=torch.float32, device=DEV)
+            kn.rope_table(freqs, i32(pos), cs)
+            extra = dict(cos_sin=cs, cu_rows=i32(cu))
+        kn.rope_store(q, k, v, heads, kv_heads, hd, freqs, i32(pos), i32(row_seq), i32(slots), table, kc, vc, BS, **extra)
+        results.append((qkv, kc, vc))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    kc, vc = results[1][1], results[1][2]
+    touched = torch.zeros((n_blocks, BS), dtype=torch.bool)
+    for b, (st, n) in enumerate(zip(starts, lens)):
+        for p in range(st, st + n):
+            touched[int(table[slots[b], p // BS]), p % BS] = True
+    assert bool((kc.cpu().permute(0, 2, 1, 3)[~touched] == 3.0).all())
+    assert bool((vc.cpu().permute(0, 3, 1, 2)[~touched] == 3.0).all())
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 33, 64, 65, 300, 400])
 @pytest.mark.parametrize("inner,k", [(16, 8), (328, 96), (1000, 264), (8200, 96), (14336, 4096), (1032, 512)])
 def test_linear_with_fused_swiglu(kn, m, inner, k):
