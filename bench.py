@@ -87,6 +87,8 @@ def main() -> int:
     ap.add_argument("--prefill-only", action="store_true", help="run the prefill alone, twice (for profiling)")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="prompt length of --prefill-only (the reported prefill is always of 2,048 tokens)")
+    ap.add_argument("--context", type=int, default=0,
+                    help="tokens a sequence may hold (default: the shape's 8192); for decoding over longer prompts")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -106,6 +108,8 @@ def main() -> int:
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
+    if args.context:
+        cfg["max_position_embeddings"] = args.context
     config = lq.LlamaConfig.from_dict(cfg)
     slot_len = cfg["max_position_embeddings"]
     max_batch = 64 if (args.shape == "8b" and not (args.no_points or args.prefill_only)) else args.batch
