@@ -99,7 +99,9 @@ class GQAttention(Mixer):
                 self.position.apply(q, k, ctx)
             if cache.write:
                 # the step's table of cos and sin, where the position encoding keeps one (the same for every layer)
-                table = self.position.cos_sin(ctx) if freqs is not None and hasattr(self.position, "cos_sin") else None
+                by_groups = getattr(kn, "rope_store_takes_table", lambda rows: False)(q.shape[0])
+                table = self.position.cos_sin(ctx) if (by_groups and freqs is not None
+                                                       and hasattr(self.position, "cos_sin")) else None
                 kn.rope_store(q, k, v, self.heads, self.kv_heads, self.head_dim, freqs, ctx.row_pos,
                               ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size,
                               cos_sin=table, cu_rows=ctx.cu_rows if table is not None else None)
