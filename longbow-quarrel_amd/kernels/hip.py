@@ -55,6 +55,9 @@ def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
     return c_void_p(0 if t is None else t.data_ptr())
 
 
+ptr = _ptr  # for parts that launch a kernel of their own through `HipKernels.call`
+
+
 def _code(t: torch.Tensor) -> int:
     try:
         return _DTYPE_CODE[t.dtype]
@@ -89,6 +92,16 @@ class HipKernels:
     def _check(self, rc: int) -> None:
         if rc != 0:
             raise KernelLibraryError(self.lib.lq_last_error().decode("utf-8", "replace"))
+
+    def call(self, symbol: str, *args) -> None:
+        """Launches an `extern "C" int symbol(..., hipStream_t)` of the library on this object's stream: for a
+        part that brings a kernel of its own (a `.hip` file beside the others is compiled into the library; the
+        function checks its arguments with LQ_REQUIRE and returns non-zero after `lq_set_error`).  `args` are
+        ctypes values; `ptr(tensor)` gives a tensor's address."""
+        fn = getattr(self.lib, symbol, None)
+        if fn is None:
+            raise KernelLibraryError(f"the kernel library has no function {symbol}")
+        self._check(fn(*args, self.stream))
 
     @staticmethod
     def _dev(*tensors: Optional[torch.Tensor]) -> None:

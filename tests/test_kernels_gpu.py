@@ -220,6 +220,21 @@ def test_products_around_a_norm(kn, m, n, k, n2):
     assert rel_err(act2, plain.swiglu(want[:, : n2 // 2], want[:, n2 // 2 :])) < 5e-3
 
 
+def test_a_library_function_called_by_name(kn):
+    """What a part with a kernel of its own uses: the function by its name, ctypes arguments, the object's
+    stream, the library's error text as an exception."""
+    from ctypes import c_int, c_longlong
+    from longbow_quarrel_amd.kernels.hip import KernelLibraryError, ptr
+    x, d = rnd((5, 77), 90), rnd((5, 77), 91)
+    want = x + d
+    kn.call("lq_add", ptr(x), ptr(d), c_int(0), c_longlong(x.numel()))
+    assert torch.equal(x, want)
+    with pytest.raises(KernelLibraryError, match="must be positive"):
+        kn.call("lq_add", ptr(x), ptr(d), c_int(0), c_longlong(0))
+    with pytest.raises(KernelLibraryError, match="no function lq_no_such_kernel"):
+        kn.call("lq_no_such_kernel")
+
+
 def test_linear_bfloat16_odd_k_takes_the_generic_kernel(kn):
     x, w = rnd((9, 77), 14, torch.bfloat16), rnd((33, 77), 15, torch.bfloat16)
     out = torch.empty((9, 33), dtype=torch.float32, device=DEV)
