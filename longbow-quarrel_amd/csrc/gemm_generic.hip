@@ -2,8 +2,8 @@
 // (internal/device/kernels.metal:105-132: "y[b,row] = sum_k W[row,k] x[b,k]").
 //
 // This file holds the size-agnostic kernel: LDS-tiled, vector FMA, 32-bit
-// accumulation, every output summed over k in ascending order, so a row's result
-// does not depend on how many other rows the launch holds.  It is the whole of
+// accumulation, every output summed over k in ascending order (in slabs of 16, each summed by
+// itself first), so a row's result does not depend on how many other rows the launch holds.  It is the whole of
 // the float32 path (no matrix-core mode that would narrow the operands) and the
 // fallback of the bfloat16 path for shapes the MFMA kernels refuse.
 #include "common.h"
@@ -46,6 +46,13 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
         Ws[lk + u][lrow] = (n < N && k0 + lk + u < K) ? to_f32(wsrc[u]) : 0.f;
     }
     __syncthreads();
+    // a slab's 16 products are summed by themselves and then added to the running sum: the rounding
+    // error of a long row grows with K / 16 + 16 additions instead of K
+    float part[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part[i][j] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < BK; ++kk) {
       float a[4], b[4];
@@ -56,8 +63,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(a[i], b[j], part[i][j]);
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] += part[i][j];
     __syncthreads();
   }
 #pragma unroll
