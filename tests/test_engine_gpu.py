@@ -423,6 +423,15 @@ def test_a_sequence_longer_than_one_split_of_decode_attention(tmp_path_factory, 
     assert rel_err(got[head:], want[head:]) < tol(dtype)
     assert rel_err(got[1020:1030], want[1020:1030]) < tol(dtype)  # the rows around the split boundary
     assert rel_err(got_short, want_short[20:]) < tol(dtype)
+    # a step of more than a thousand rows (in bfloat16 the rotation then takes eight positions a workgroup):
+    # one sequence goes on from position 5, the other starts beside it
+    eng.release(a)
+    eng.release(b)
+    a, b = eng.new_sequence(), eng.new_sequence()
+    first = eng.step([StepEntry(a, req[:5], range(5))])
+    rest = eng.step([StepEntry(a, req[5:], range(n - 5)), StepEntry(b, short, range(len(short)))])
+    assert rel_err(torch.cat([first, rest[: n - 5]]), want) < tol(dtype)
+    assert rel_err(rest[n - 5 :], want_short) < tol(dtype)
 
 
 def test_generation_through_graphs_on_the_matrix_core_decode_path_across_a_length_bucket(tmp_path_factory):
