@@ -20,13 +20,18 @@ class SamplerConfig:
     """Zero values mean what they mean in the reference: temperature 0 is greedy
     (internal/engine/sampler.go:81-84), top_k <= 0 and top_p <= 0 or >= 1 are off (:309-339),
     rep_penalty acts above 1 (:77-79).  Only the seed differs: 0 is a seed like any other here,
-    the reference takes the clock for it (:18-26)."""
+    the reference takes the clock for it (:18-26).  `debug_activations` and `quality_mode` are the
+    reference's remaining two fields (internal/engine/types_base.go:13-14): the first makes it log
+    statistics of activations, which `Engine.step(observe=...)` and `trace_run --dump-activations` give
+    as tensors here, the second is never read there; both are accepted and change nothing."""
 
     temperature: float = 0.0
     top_k: int = 0
     top_p: float = 0.0
     rep_penalty: float = 0.0
     seed: int = 0
+    debug_activations: bool = False
+    quality_mode: bool = False
 
     def params(self) -> SamplingParams:
         return SamplingParams(temperature=self.temperature, top_k=max(0, self.top_k),
