@@ -167,6 +167,7 @@ struct AttnArgs {
   float* part_ml;  // [rows][nh][nsplit][2]
   int nsplit;
   int split_len;   // positions per split, a multiple of 256
+  int units;       // > 0: workgroups a kv head, which share the sequences' splits out among themselves
   int* tickets;    // [rows][nkv], zero between launches: how many splits of the row have finished
   // decode with the rotation and the cache write folded in (all null otherwise): the step's
   // unrotated keys and values, and cos/sin of every row's angles [rows][HD/2][2]
@@ -747,6 +748,67 @@ int launch_rows32(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
 // ------------------------------------------------------------------ heads (decoding)
 // Block = NW waves over one split of one (sequence, kv head).  LDS: per wave HD x G floats of
 // partial output (the valid columns only), G maxima, G normalisers.
+// Which split of which sequence unit u of a kv head takes, when the units share the work out themselves
+// (a few sequences, no window).  Every sequence's keys are cut into splits of one length: the smallest
+// multiple of 256 with which the splits that hold keys number no more than the launch has units for a kv
+// head.  Those splits are numbered through, sequence after sequence, and unit u takes number u.  With
+// sequences of unequal lengths a launch whose grid is (sequence, split) leaves the splits of the short ones
+// empty and makes the long ones' as large as if all were long; here a unit has work or ends at once, and
+// the units with work follow one another, so that the compute units (which take workgroups in turn) get
+// equal numbers of them.  Lane l holds sequence l; every wave of the workgroup works out the same answer.
+struct DecodeItem {
+  int row, pos, slot, split_len, split;
+  int first_unit, n_full, last_unit;  // the row's whole splits sit in units first_unit .., its last, part-filled one in last_unit
+};
+
+// Inclusive prefix sums over the wave's 64 lanes with data-parallel-primitive moves (no trip through LDS):
+// within rows of 16 lanes by shifts of 1, 2, 4 and 8 (lanes shifted in from outside a row read zero), then
+// lane 15 of a row into the odd rows and lane 31 into the upper half.
+__device__ inline int wave_prefix_sums(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+__device__ inline bool balanced_item(const AttnArgs& a, int u, DecodeItem& it) {
+  const int lane = threadIdx.x & 63;
+  const bool mine = lane < a.batch;
+  const int pl = mine ? a.row_pos[lane] : -1;  // lane l looks after sequence l (at most 32 of them)
+  const int sl = mine ? a.seq_slot[lane] : 0;
+  const int total = __builtin_amdgcn_readlane(wave_prefix_sums(pl + 1), 63);
+  // the smallest multiple of 256 with which the splits that hold keys are no more than the units; blocks of
+  // 256 positions and their quotients are small integers, which a float division gives exactly
+  const float blocks = (float)(pl >> 8) + 0.5f;  // (position p lies in block p / 256)
+  int k = max(1, (total + 256 * a.units - 1) / (256 * a.units)), cnt = 0;
+  for (int tries = 0; tries < 1024; ++tries, ++k) {
+    cnt = mine ? (int)(blocks / (float)k) + 1 : 0;  // splits of this lane's sequence that hold keys
+    if (__builtin_amdgcn_readlane(wave_prefix_sums(cnt), 63) <= a.units) break;
+  }
+  const int SL = 256 * k;
+  // whole splits first, sequence after sequence, then the last splits (the part-filled ones): the two
+  // workgroups that share a compute unit, c and c + 32 of a die's run, then differ as little as may be
+  const int part = mine && (pl + 1) % SL != 0 ? 1 : 0, full = cnt - part;
+  const int full_incl = wave_prefix_sums(full), part_incl = wave_prefix_sums(part);
+  const int n_full = __builtin_amdgcn_readlane(full_incl, 63), n_part = __builtin_amdgcn_readlane(part_incl, 63);
+  if (n_full + n_part > a.units || u >= n_full + n_part) return false;  // (the first cannot be: see decode_units)
+  const bool whole = u < n_full;
+  const int row = whole ? __popcll(__ballot(mine && full_incl <= u))
+                        : __popcll(__ballot(mine && part_incl <= u - n_full));
+  it.row = row;
+  it.pos = __builtin_amdgcn_readlane(pl, row);
+  it.slot = __builtin_amdgcn_readlane(sl, row);
+  it.split_len = SL;
+  it.n_full = __builtin_amdgcn_readlane(full, row);
+  it.first_unit = __builtin_amdgcn_readlane(full_incl - full, row);
+  it.last_unit = n_full + __builtin_amdgcn_readlane(part_incl - part, row);
+  it.split = whole ? u - it.first_unit : it.n_full;
+  return true;
+}
+
 template <int HD, int NW>
 __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -754,14 +816,30 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kerne
   float* lds_o = lds;                    // [NW][HD][G]
   float* lds_m = lds + NW * HD * G;      // [NW][G]
   float* lds_l = lds_m + NW * G;         // [NW][G]
-  const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, g = lane >> 4;
+  // grid (sequence, kv head, split), or (kv head, unit) when the units share the splits out themselves
+  int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, SL = a.split_len, p, slot;
+  int first_unit = 0, n_full = 0, last_unit = 0;
+  if (a.units > 0) {
+    DecodeItem it;
+    kvh = blockIdx.x;
+    if (!balanced_item(a, blockIdx.y, it)) return;  // the whole block: more units than splits with keys
+    b = it.row;
+    p = it.pos;
+    slot = it.slot;
+    SL = it.split_len;
+    split = it.split;
+    first_unit = it.first_unit;
+    n_full = it.n_full;
+    last_unit = it.last_unit;
+  } else {
+    p = a.row_pos[b];
+    slot = a.seq_slot[b];
+  }
   const int r = b;  // a decoding step has one row a sequence, in the order of the sequences
-  // Everything that depends on the row alone is asked for at once, before the position is known:
-  // a block's time is a chain of memory round trips (position, block table, keys), and these join
-  // the first of them.
-  const int p = a.row_pos[r];
-  const int slot = a.seq_slot[b];
+  // Everything that depends on the row alone is asked for at once, before the position is known
+  // (or, with units, together with the block table): a block's time is a chain of memory round trips
+  // (position, block table, keys), and these join the first of them.
   const int h = kvh * G + min(c16, G - 1);
   const bool folded = HD % 64 == 0 && a.cs != nullptr;
   u32x4 qraw[HD / 32];
@@ -814,7 +892,7 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kerne
     }
   }
   const int lo = (a.window > 0 && p >= a.window) ? p - a.window + 1 : 0;
-  const int SL = a.split_len, lo64 = (lo / BS) * BS;
+  const int lo64 = (lo / BS) * BS;
   const int s_begin = max(split * SL, lo64);
   const int s_end = min(split * SL + SL - 1, p);
   if (s_begin > s_end) return;  // the whole block: this split holds no key of the row
@@ -896,11 +974,13 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kerne
     if (s_first == s_last) {
       a.out[(long long)r * a.ldo + hh * HD + d] = f32_to_bf16(acc / L);
     } else {
-      const long long slot = ((long long)r * a.nh + hh) * a.nsplit + split;
-      publish_result(a.part_o + slot * HD + d, acc);
+      // a split's partial results lie by (row, head, split), or by (kv head, unit, head of the group)
+      const long long at = a.units > 0 ? ((long long)kvh * a.units + (split < n_full ? first_unit + split : last_unit)) * G + c
+                                       : ((long long)r * a.nh + hh) * a.nsplit + split;
+      publish_result(a.part_o + at * HD + d, acc);
       if (d == 0) {
-        publish_result(a.part_ml + slot * 2, M);
-        publish_result(a.part_ml + slot * 2 + 1, L);
+        publish_result(a.part_ml + at * 2, M);
+        publish_result(a.part_ml + at * 2 + 1, L);
       }
     }
   }
@@ -921,7 +1001,11 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kerne
   for (int idx = threadIdx.x; idx < HD * G; idx += NW * 64) {
     const int d = idx / G, c = idx - d * G;
     const int hh = kvh * G + c;
-    const long long base = ((long long)r * a.nh + hh) * a.nsplit;
+    // split s of the row lies at place(s): by (row, head, split), or by (kv head, unit, head of the group)
+    auto place = [&](int sidx) -> long long {
+      if (a.units > 0) return ((long long)kvh * a.units + (sidx < n_full ? first_unit + sidx : last_unit)) * G + c;
+      return ((long long)r * a.nh + hh) * a.nsplit + sidx;
+    };
     // four splits' values are asked for together; the sum runs in ascending split order under a
     // running maximum
     float M = -INFINITY, acc = 0.f, L = 0.f;
@@ -929,7 +1013,7 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kerne
       float pm[4], pl[4], po[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const long long sp = base + min(s0 + j, s_last);
+        const long long sp = place(min(s0 + j, s_last));
         pm[j] = other_blocks_result(a.part_ml + sp * 2);
         pl[j] = other_blocks_result(a.part_ml + sp * 2 + 1);
         po[j] = other_blocks_result(a.part_o + sp * HD + d);
@@ -978,6 +1062,7 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
   // of which a compute unit holds several, each wave with one chunk in flight.
   const int per_wave = (HD * G + 2 * G) * (int)sizeof(float);
   dim3 grid(a.batch, a.nkv, a.nsplit);
+  if (a.units > 0) grid = dim3(a.nkv, a.units, 1);
   if (4 * per_wave <= 48 * 1024)
     attn_heads_kernel<HD, 4><<<grid, 4 * 64, (size_t)4 * per_wave, stream>>>(a);
   else
@@ -1006,11 +1091,25 @@ static int decode_split_len(int rows, int nkv, int max_len) {
   return (int)(256 * (per > 1 ? per : 1));
 }
 
-// Floats of workspace a decode launch needs (0 when one split is enough).
+// Units a kv head for a decoding launch whose workgroups share the splits out themselves (0: the grid is
+// (sequence, kv head, split)): as many as keep the launch within MAX_DECODE_BLOCKS workgroups, no more than
+// the sequences have splits of 256 within their bound, and at least two a sequence.  Taken for 2 to 32
+// sequences without a window.
+static int decode_units(int rows, int nkv, int max_len, int window) {
+  if (window > 0 || rows < 2 || rows > 32) return 0;
+  const long long bound = (long long)lq_ceil_div(max_len, 1024) * 1024;
+  const long long by_cap = MAX_DECODE_BLOCKS / nkv, by_bound = (long long)rows * (bound / 256);
+  const long long units = by_cap < by_bound ? by_cap : by_bound;
+  return units >= 2 * rows ? (int)units : 0;
+}
+
+// Floats of workspace a decode launch needs (0 when one split is enough): enough for either grid, the
+// window being unknown here.
 long long lq_attention_mfma_workspace(int rows, int nh, int nkv, int hd, int max_len) {
   const int nsplit = lq_ceil_div(max_len, decode_split_len(rows, nkv, max_len));
-  if (nsplit <= 1) return 0;
-  return (long long)rows * nh * nsplit * (hd + 2);
+  const long long classic = nsplit <= 1 ? 0 : (long long)rows * nh * nsplit * (hd + 2);
+  const long long shared = (long long)decode_units(rows, nkv, max_len, 0) * nh * (hd + 2);
+  return classic > shared ? classic : shared;
 }
 
 int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int batch, int nh, int nkv,
@@ -1018,7 +1117,7 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
                       const int* block_table, int bt_stride, const void* kcache, const void* vcache,
                       float scale, int window, int decode, int max_len, float* workspace,
                       long long workspace_floats, int* tickets, long long tickets_n, const void* k_new,
-                      const void* v_new, int ldk, int ldv, const float* cs, hipStream_t stream) {
+                      const void* v_new, int ldk, int ldv, const float* cs, int uneven, hipStream_t stream) {
   AttnArgs a;
   a.q = (const bf16_t*)q;
   a.ldq = ldq;
@@ -1040,6 +1139,7 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
   a.part_ml = nullptr;
   a.nsplit = 1;
   a.split_len = 256;
+  a.units = 0;
   a.tickets = tickets;
   a.k_new = (const bf16_t*)k_new;
   a.v_new = (const bf16_t*)v_new;
@@ -1057,7 +1157,17 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
     a.split_len = decode_split_len(rows, nkv, max_len);
     a.nsplit = lq_ceil_div(max_len, a.split_len);
     LQ_REQUIRE(a.nsplit <= 65535, "attention: %d tokens are too many splits", max_len);
-    if (a.nsplit > 1) {
+    a.units = uneven && max_len > 256 ? decode_units(rows, nkv, max_len, window) : 0;
+    if (a.units > 0) {
+      const long long need = (long long)a.units * nh * (hd + 2);
+      LQ_REQUIRE(workspace != nullptr && workspace_floats >= need,
+                 "attention: workspace of %lld floats needed, %lld given", need, workspace_floats);
+      LQ_REQUIRE(tickets != nullptr && tickets_n >= (long long)rows * nkv,
+                 "attention: %lld ticket counters needed for %d rows and %d kv heads, %lld given",
+                 (long long)rows * nkv, rows, nkv, tickets_n);
+      a.part_o = workspace;
+      a.part_ml = workspace + (long long)a.units * nh * hd;
+    } else if (a.nsplit > 1) {
       const long long need = lq_attention_mfma_workspace(rows, nh, nkv, hd, max_len);
       LQ_REQUIRE(workspace != nullptr && workspace_floats >= need,
                  "attention: workspace of %lld floats needed, %lld given", need, workspace_floats);

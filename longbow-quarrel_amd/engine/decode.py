@@ -37,10 +37,12 @@ def _pad4(n: int) -> int:
 
 
 class DecodeGraph:
-    def __init__(self, engine, batch: int, bound: int, ws: Workspace, logits: torch.Tensor) -> None:
+    def __init__(self, engine, batch: int, bound: int, ws: Workspace, logits: torch.Tensor,
+                 uneven: bool = False) -> None:
         self.engine = engine
         self.batch = batch
         self.bound = bound
+        self.uneven = uneven  # the step's hint to the attention kernel (`lengths_uneven`), fixed at capture
         dev = engine.device
         b = batch
         self.sizes = [b, b, b, b, b, b, b + 1, b]  # tokens row_seq row_pos slot start len cu want
@@ -77,7 +79,7 @@ class DecodeGraph:
         e = self.engine
         return e.make_context(self.ws, self.views[:7], self.slots or [0] * self.batch, [], [1] * self.batch,
                               self.bound, logits_out=self.logits,
-                              kernels=DryKernels(e.kernels) if dry else None, dry=dry)
+                              kernels=DryKernels(e.kernels) if dry else None, dry=dry, uneven=self.uneven)
 
     def run_body(self, sampler: Sampler) -> None:
         """What one decoding step launches; the same calls whether captured or run directly."""
@@ -114,8 +116,8 @@ class DecodeGraph:
 
 
 class DecodeGraphs:
-    """The captured decoding steps of one backend, keyed by (batch size, length bound), and the
-    workspace and logits buffer that they share."""
+    """The captured decoding steps of one backend, keyed by (batch size, length bound, whether the
+    lengths are uneven), and the workspace and logits buffer that they share."""
 
     graph_cls = DecodeGraph
 
@@ -124,13 +126,13 @@ class DecodeGraphs:
         self.sampler = sampler
         self.ws = Workspace(engine.device, 1 << 16)
         self.logits: Optional[torch.Tensor] = None
-        self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}
+        self.graphs: Dict[Tuple[int, int, bool], DecodeGraph] = {}
         self.captures = 0
 
-    def get(self, batch: int, bound: int) -> Tuple[DecodeGraph, bool]:
-        """The graph for this batch size and bound, and whether it is new (then the caller loads its
+    def get(self, batch: int, bound: int, uneven: bool = False) -> Tuple[DecodeGraph, bool]:
+        """The graph for this batch size, bound and hint, and whether it is new (then the caller loads its
         arrays and calls `capture`)."""
-        key = (batch, bound)
+        key = (batch, bound, bool(uneven))
         g = self.graphs.get(key)
         if g is not None:
             return g, False
@@ -138,7 +140,7 @@ class DecodeGraphs:
         if self.logits is None or self.logits.shape[0] < batch:
             self.drop_all()
             self.logits = torch.empty((batch, e.vocab_size), dtype=torch.float32, device=e.device)
-        g = self.graph_cls(e, batch, bound, self.ws, self.logits[:batch])
+        g = self.graph_cls(e, batch, bound, self.ws, self.logits[:batch], bool(uneven))
         self.ws.frozen = False
         if not g.walk():
             self.drop_all()  # the buffers are about to move: the graphs that point into them go

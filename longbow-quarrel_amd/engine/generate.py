@@ -36,7 +36,7 @@ from ..sampling.params import SamplingParams
 from ..sampling.sampler import NonFiniteLogits, Sampler
 from ..sampling.state import SamplerState, sequence_key
 from .decode import LEN_BUCKET, DecodeGraphs
-from .step import Engine, SequenceTooLong, StepEntry
+from .step import Engine, SequenceTooLong, StepEntry, lengths_uneven
 
 
 @dataclass
@@ -341,8 +341,9 @@ class EngineBackend:
         longest = max(starts) + 1
         bound = (longest + LEN_BUCKET - 1) // LEN_BUCKET * LEN_BUCKET
         growth = {s: 1 for s in slots}
+        uneven = lengths_uneven([n + 1 for n in starts])
         if same_graph is not None:
-            if bound != same_graph.bound:
+            if bound != same_graph.bound or uneven != same_graph.uneven:
                 return None
             try:
                 for s, n in zip(slots, starts):
@@ -355,7 +356,7 @@ class EngineBackend:
             for s, n in zip(slots, starts):
                 e.check_room(s, n, 1)
             cache.reserve(growth)
-            g, fresh = self.graphs.get(len(slots), bound)
+            g, fresh = self.graphs.get(len(slots), bound, uneven)
             # a graph's arrays carry on from its own last step only: anything else in between (another graph,
             # a prompt step, a batch whose members changed) means they are written anew
             if fresh or changed or g is not self.current or g.slots != slots:

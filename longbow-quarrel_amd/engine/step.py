@@ -28,6 +28,14 @@ from ..model import DecoderModel
 from ..parts.base import BuildEnv, StepContext, Workspace
 
 
+def lengths_uneven(lengths: Sequence[int]) -> bool:
+    """Whether the sequences of a decoding step differ so much in length (the longest at least half again
+    as long as their mean) that the attention kernel does better sharing the keys out by the true lengths
+    than cutting every sequence as if it were the longest.  The one place where this is decided, for direct
+    and for captured steps alike, so that both sum in the same order."""
+    return len(lengths) >= 2 and 2 * len(lengths) * max(lengths) >= 3 * sum(lengths)
+
+
 class SequenceTooLong(ValueError):
     """A step would take a sequence past `Engine.max_sequence_tokens`."""
 
@@ -168,19 +176,19 @@ class Engine:
 
     def make_context(self, ws: Workspace, arrays: Sequence[torch.Tensor], slots: Sequence[int],
                      starts: Sequence[int], new: Sequence[int], max_len: int, logits_out=None, observe=None,
-                     kernels=None, dry: bool = False) -> StepContext:
+                     kernels=None, dry: bool = False, uneven: bool = False) -> StepContext:
         """The one place where a step's `StepContext` is put together, for direct and for captured steps.
         `arrays`: the device arrays tokens, row_seq, row_pos, seq_slot, seq_start, seq_len, cu_rows;
         `slots`, `starts`, `new`: per sequence, on the host (`starts` may be empty where the lengths
         live on the device only, as in a captured step); `max_len`: an upper bound of the lengths after
-        the step."""
+        the step; `uneven`: whether a decoding step's sequences differ much in length (`lengths_uneven`)."""
         tokens, row_seq, row_pos, seq_slot, seq_start, seq_len, cu_rows = arrays
         return StepContext(
             kernels=kernels if kernels is not None else self.kernels, dtype=self.dtype, device=self.device, ws=ws,
             rows=sum(new), batch=len(new), tokens=tokens, row_seq=row_seq, row_pos=row_pos, seq_slot=seq_slot,
             seq_start=seq_start, seq_len=seq_len, cu_rows=cu_rows, host_slots=list(slots), host_start=list(starts),
             host_new=list(new), max_new=max(new), max_len=max_len, decode=all(n == 1 for n in new),
-            logits_out=logits_out, observe=observe, dry=dry)
+            logits_out=logits_out, observe=observe, dry=dry, uneven=uneven and all(n == 1 for n in new))
 
     def forward(self, ctx: StepContext, want_rows: torch.Tensor, n_want: int) -> Optional[torch.Tensor]:
         """The model over one step's rows, from this engine's cache."""
@@ -213,7 +221,8 @@ class Engine:
 
         self.ws.reset()
         ctx = self.make_context(self.ws, (d_tokens, d_row_seq, d_row_pos, d_slot, d_start, d_len, d_cu), slots,
-                                starts, [len(e.tokens) for e in entries], max(lens), observe=observe)
+                                starts, [len(e.tokens) for e in entries], max(lens), observe=observe,
+                                uneven=lengths_uneven(lens))
         logits = self.forward(ctx, d_want, len(want_rows))
         cache.advance(growth)
         self.steps_run += 1

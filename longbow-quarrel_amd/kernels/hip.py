@@ -20,6 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
+ABI_VERSION = 2  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -47,6 +48,9 @@ def load_library() -> ctypes.CDLL:
         raise KernelLibraryError(f"cannot load {path}: {e}") from e
     lib.lq_last_error.restype = ctypes.c_char_p
     lib.lq_abi_version.restype = c_int
+    if lib.lq_abi_version() != ABI_VERSION:
+        raise KernelLibraryError(f"{path} speaks version {lib.lq_abi_version()} of the kernel interface, "
+                                 f"this package version {ABI_VERSION}: build it again")
     _LIB = lib
     return lib
 
@@ -432,11 +436,14 @@ class HipKernels:
                   block_table: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                   block_size: int, scale: float, window: int = 0, decode: bool = False, max_len: int = 0,
                   workspace: Optional[torch.Tensor] = None, k_new: Optional[torch.Tensor] = None,
-                  v_new: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None) -> None:
+                  v_new: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None,
+                  uneven: bool = False) -> None:
         """Causal grouped-query attention of the step's rows over their slots' cached keys.
 
         `decode` promises one row per sequence; `max_len` is then an upper bound of the lengths
         after this step and `workspace` float32 scratch of `attention_workspace(...)` entries.
+        `uneven` says that the sequences of a decoding step differ much in length (the step's
+        context knows): the launch then shares the keys out over its workgroups by the true lengths.
         With `cos_sin` (a `rope_table` of this step; only where `attention_folds_rope` says so) q, k_new
         and v_new are the unrotated projections: the launch rotates q and k and writes k and v into
         the cache itself."""
@@ -483,7 +490,7 @@ class HipKernels:
             c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
             c_longlong(ws_n), _ptr(self._tickets), c_longlong(self._tickets.numel()), _ptr(k_new if cos_sin is not None else None),
             _ptr(v_new if cos_sin is not None else None), c_int(ldk), c_int(ldv), _ptr(cos_sin),
-            c_int(1 if self.force_generic else 0), self.stream)
+            c_int(1 if uneven and decode else 0), c_int(1 if self.force_generic else 0), self.stream)
         if rc != 0:
             # a launch that did not run whole may have left tickets behind, and a later launch that found
             # them non-zero would never recognise its last workgroup: clear them (a fill kernel) before

@@ -93,7 +93,7 @@ class GQAttention(Mixer):
             kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
                          ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
                          self.scale, self.window, decode=True, max_len=ctx.max_len, workspace=scratch,
-                         k_new=k, v_new=v, cos_sin=self.position.cos_sin(ctx))
+                         k_new=k, v_new=v, cos_sin=self.position.cos_sin(ctx), uneven=ctx.uneven)
         else:
             if freqs is None:
                 self.position.apply(q, k, ctx)
@@ -109,5 +109,6 @@ class GQAttention(Mixer):
                 kn.rope_store(q, None, None, self.heads, 0, self.head_dim, freqs, ctx.row_pos)
             kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
                          ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
-                         self.scale, self.window, decode=ctx.decode, max_len=ctx.max_len, workspace=scratch)
+                         self.scale, self.window, decode=ctx.decode, max_len=ctx.max_len, workspace=scratch,
+                         uneven=ctx.uneven)
         return project_into(kn, ctx, att, self.w_o, sink)

@@ -251,6 +251,9 @@ class StepContext:
     max_new: int = 0
     max_len: int = 0
     decode: bool = False  # every sequence brings exactly one token
+    # a decoding step whose sequences differ much in length (`lengths_uneven`): a hint, which changes how the
+    # attention kernel shares its work out and nothing in the result beyond the order of its sums
+    uneven: bool = False
     logits_out: Optional[torch.Tensor] = None  # where the logits go (a captured step's fixed buffer)
     # True while a step is only walked through to learn its workspace size: `kernels` then answers
     # size questions and launches nothing; a part that launches kernels of its own must not either

@@ -111,7 +111,7 @@ class CpuKernels:
         return 0
 
     def attention(self, q, out, heads, kv_heads, head_dim, row_pos, row_seq, seq_slot, cu_rows, block_table,
-                  kcache, vcache, block_size, scale, window=0, decode=False, max_len=0, workspace=None):
+                  kcache, vcache, block_size, scale, window=0, decode=False, max_len=0, workspace=None, uneven=False):
         rows = q.shape[0]
         group = heads // kv_heads
         for r in range(rows):

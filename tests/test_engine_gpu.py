@@ -461,7 +461,7 @@ def test_generation_through_graphs_on_the_matrix_core_decode_path_across_a_lengt
         res = GenerationLoop(be, max_batch=3).run(prompts, 70, stop_ids=[], callback=callback)
         if graphs:
             # the second graph's attention needs more workspace than the first had: the first one went
-            assert (3, 2048) in be.graphs.graphs and be.graphs.captures == 2
+            assert (3, 2048, False) in be.graphs.graphs and be.graphs.captures == 2
         be.close()
         runs[graphs] = (res.tokens, torch.stack(seen))
     assert runs[True][0] == runs[False][0] and all(len(t) == 70 for t in runs[True][0])
@@ -471,6 +471,71 @@ def test_generation_through_graphs_on_the_matrix_core_decode_path_across_a_lengt
     want = ref.forward(seq[:1040], plain.round_bf16)
     for k in range(15, 35):
         assert rel_err(runs[True][1][k], want[1000 + k - 1]) < TOL_BF16, k
+    assert eng.cache.slots.taken_count == 0
+
+
+def test_generation_with_sequences_of_very_unequal_lengths(tmp_path_factory):
+    """Prompts of 1 400, 300, 290 and 310 tokens in one batch on the 8B head shape: the decoding steps tell the
+    attention kernel that the lengths are uneven, and it shares the long sequence's keys out over the
+    workgroups that the short ones leave free.  The hint reaches the kernel in captured and in direct steps
+    alike (the tokens and the logits of both are equal), the logits agree with the plain implementation, and
+    once the long sequence has ended the rest goes on without the hint."""
+    from longbow_quarrel_amd.engine.generate import EngineBackend, GenerationLoop
+    from longbow_quarrel_amd.engine.step import lengths_uneven
+
+    assert lengths_uneven([1401, 61, 26, 301]) and not lengths_uneven([530] * 8) and not lengths_uneven([900])
+    assert not lengths_uneven([1000, 985, 300]) and lengths_uneven([3000, 1000])
+    folder = write_folder(tmp_path_factory.mktemp("uneven"), LONG, seed=10, std=0.08)
+    c, tensors = read_folder(folder)
+    ref = plain.PlainLlama(c, tensors)
+    eng = lq.load_engine(folder, dtype="bfloat16", max_tokens=4096)
+    kn = eng.kernels
+    prompts = [random_tokens(n, LONG["vocab_size"], 800 + n) for n in (300, 290, 310, 1400)]
+    hints = []
+    attention = kn.attention
+
+    def watched(*a, **k):
+        if k.get("decode"):
+            hints.append(bool(k.get("uneven")))
+        return attention(*a, **k)
+
+    runs = {}
+    kn.attention = watched
+    try:
+        for graphs in (False, True):
+            be = EngineBackend(eng, lq.SamplingParams(), use_graphs=graphs)
+            be.keep_logits = True
+            seen, seen_long = [], []
+
+            def callback(request, token, be=be, seen=seen, seen_long=seen_long):
+                if request == 0:
+                    seen.append(be.last_logits[0].clone())
+                if request == 3:  # (the last row for as long as it lives)
+                    seen_long.append(be.last_logits[3].clone())
+
+            del hints[:]
+            # the long request may take 12 tokens, the others 30: the last 18 steps hold three short sequences
+            loop = GenerationLoop(be, max_batch=4)
+            limits = loop._token_limits
+            loop._token_limits = lambda prompts, n: [12 if len(p) > 1000 else n for p in prompts]
+            res = loop.run(prompts, 30, stop_ids=[], callback=callback)
+            be.close()
+            runs[graphs] = (res.tokens, torch.stack(seen), list(hints), torch.stack(seen_long))
+    finally:
+        kn.attention = attention
+    assert runs[True][0] == runs[False][0] and [len(t) for t in runs[True][0]] == [30, 30, 30, 12]
+    assert torch.equal(runs[True][1], runs[False][1])
+    assert any(runs[False][2]) and not all(runs[False][2])  # with the long sequence, and without it
+    assert any(runs[True][2]) and not all(runs[True][2])    # (captured steps: the calls of the captures)
+    seq = prompts[0] + runs[True][0][0]
+    want = ref.forward(seq, plain.round_bf16)
+    for k in range(1, 30):  # request 0 holds 300 + k tokens when its token k + 1 is sampled
+        assert rel_err(runs[True][1][k], want[300 + k - 1]) < TOL_BF16, k
+    long_seq = prompts[3] + runs[True][0][3]
+    want_long = ref.forward(long_seq, plain.round_bf16)
+    assert torch.equal(runs[True][3], runs[False][3])
+    for k in range(1, 12):  # the long request, whose keys the workgroups share out
+        assert rel_err(runs[True][3][k], want_long[1400 + k - 1]) < TOL_BF16, k
     assert eng.cache.slots.taken_count == 0
 
 

@@ -283,7 +283,7 @@ def paged_cache(lengths, kv_heads, head_dim, dtype, seed):
 
 
 def run_attention(kn, q_rows, lengths, new, heads, kv_heads, head_dim, dtype, seed, window=0, decode=False,
-                  force_generic=False, standout=None, max_len=None):
+                  force_generic=False, standout=None, max_len=None, uneven=False):
     """q rows for the last `new[b]` positions of each sequence; returns (got, want)."""
     kc, vc, table, slots, dense = paged_cache(lengths, kv_heads, head_dim, dtype, seed)
     g = torch.Generator().manual_seed(seed + 1)
@@ -314,7 +314,7 @@ def run_attention(kn, q_rows, lengths, new, heads, kv_heads, head_dim, dtype, se
         need = kn.attention_workspace(dtype, rows, heads, kv_heads, head_dim, BS, decode, max_len)
         ws = torch.empty(need, dtype=torch.float32, device=DEV) if need else None
         kn.attention(qd, out, heads, kv_heads, head_dim, i32(row_pos), i32(row_seq), i32(slots), i32(cu),
-                     table, kc, vc, BS, scale, window, decode=decode, max_len=max_len, workspace=ws)
+                     table, kc, vc, BS, scale, window, decode=decode, max_len=max_len, workspace=ws, uneven=uneven)
     finally:
         kn.force_generic = False
     want = torch.zeros((rows, heads, head_dim), dtype=torch.float64)
@@ -516,6 +516,37 @@ def test_rope_store_by_groups_of_eight_positions_writes_the_same_bits(kn, heads,
             touched[int(table[slots[b], p // BS]), p % BS] = True
     assert bool((kc.cpu().permute(0, 2, 1, 3)[~touched] == 3.0).all())
     assert bool((vc.cpu().permute(0, 3, 1, 2)[~touched] == 3.0).all())
+
+
+@pytest.mark.parametrize("head_dim,heads,kv_heads,lengths", [
+    (128, 8, 2, [5000, 300, 40, 1025, 256, 257, 2, 3000]),            # one long sequence among short ones
+    (64, 4, 1, [700, 64, 1, 1500, 1500, 513, 30, 31, 32, 33, 9000]),  # one kv head; 11 sequences
+    (128, 4, 4, [600, 4700]),                                         # two sequences, no head shared
+    (192, 6, 3, [2500, 10, 900]),                                     # (two waves a workgroup)
+    (64, 8, 2, [260] * 3 + [3000] * 2 + [1] * 27),                    # 32 sequences, most of one token
+])
+def test_decode_attention_that_shares_its_keys_out_by_the_true_lengths(kn, head_dim, heads, kv_heads, lengths):
+    """With the hint that the lengths are uneven the workgroups of a decoding launch number the splits that hold
+    keys through (whole splits first, then every sequence's last) and each takes one, whatever sequence it belongs
+    to: against the plain implementation, against the launch without the hint (the same sums in another order),
+    twice the same, the tickets back at zero; a far key that stands out is found in the long sequence."""
+    n = len(lengths)
+    got, want = run_attention(kn, None, lengths, [1] * n, heads, kv_heads, head_dim, torch.bfloat16, 41, decode=True,
+                              uneven=True)
+    assert rel_err(got, want) < 8e-3
+    for b in range(n):  # every sequence by itself: a short one is not hidden behind a long one's size
+        assert rel_err(got[b], want[b]) < 1.2e-2, b
+    plain_grid, _ = run_attention(kn, None, lengths, [1] * n, heads, kv_heads, head_dim, torch.bfloat16, 41, decode=True)
+    assert rel_err(got, plain_grid.double().cpu()) < 8e-3
+    again, _ = run_attention(kn, None, lengths, [1] * n, heads, kv_heads, head_dim, torch.bfloat16, 41, decode=True,
+                             uneven=True)
+    assert torch.equal(got, again)
+    assert int(kn._tickets.abs().max()) == 0
+    longest = max(range(n), key=lambda b: lengths[b])
+    got, want = run_attention(kn, None, lengths, [1] * n, heads, kv_heads, head_dim, torch.bfloat16, 43, decode=True,
+                              uneven=True, standout=(longest, 77))
+    assert rel_err(got, want) < 8e-3
+    assert float(got[longest].float().mean()) > 6.0  # the values of key 77 (7.0) dominate the long sequence's row
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 33, 64, 65, 300, 400])
