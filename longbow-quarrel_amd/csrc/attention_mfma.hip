@@ -751,11 +751,12 @@ int launch_rows32(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
 // Which split of which sequence unit u of a kv head takes, when the units share the work out themselves
 // (a few sequences, no window).  Every sequence's keys are cut into splits of one length: the smallest
 // multiple of 256 with which the splits that hold keys number no more than the launch has units for a kv
-// head.  Those splits are numbered through, sequence after sequence, and unit u takes number u.  With
-// sequences of unequal lengths a launch whose grid is (sequence, split) leaves the splits of the short ones
-// empty and makes the long ones' as large as if all were long; here a unit has work or ends at once, and
-// the units with work follow one another, so that the compute units (which take workgroups in turn) get
-// equal numbers of them.  Lane l holds sequence l; every wave of the workgroup works out the same answer.
+// head.  Those splits are numbered through (the whole ones first, sequence after sequence, then every
+// sequence's last, part-filled one), and unit u takes number u.  With sequences of unequal lengths a launch
+// whose grid is (sequence, split) leaves the splits of the short ones empty and makes the long ones' as large
+// as if all were long; here a unit has work or ends at once, and the units with work follow one another, so
+// that the compute units (which take workgroups in turn) get equal numbers of them.  Lane l holds sequence l;
+// every wave of the workgroup works out the same answer.
 struct DecodeItem {
   int row, pos, slot, split_len, split;
   int first_unit, n_full, last_unit;  // the row's whole splits sit in units first_unit .., its last, part-filled one in last_unit
@@ -1100,7 +1101,12 @@ static int decode_units(int rows, int nkv, int max_len, int window) {
   const long long bound = (long long)lq_ceil_div(max_len, 1024) * 1024;
   const long long by_cap = MAX_DECODE_BLOCKS / nkv, by_bound = (long long)rows * (bound / 256);
   const long long units = by_cap < by_bound ? by_cap : by_bound;
-  return units >= 2 * rows ? (int)units : 0;
+  if (units < 2 * rows) return 0;
+  // The split length is looked for upwards from (all keys) / (256 units) and found before twice that: with at
+  // least two units a sequence, splits of 2 (all keys) / units leave every sequence one to spare.  The kernel
+  // gives the search 1 024 steps.
+  if (rows * bound / (256 * units) > 512) return 0;
+  return (int)units;
 }
 
 // Floats of workspace a decode launch needs (0 when one split is enough): enough for either grid, the
