@@ -25,11 +25,16 @@
 //    `split_len` positions in turn (wave w: blocks w, w + NW, ...) and combine their partial results
 //    through LDS in wave order.  A compute unit keeps about a hundred memory requests in flight,
 //    whatever their size, so a sequence's keys are spread over many workgroups: a split is 256
-//    positions unless that would make more than MAX_DECODE_BLOCKS workgroups.  A row with several
+//    positions or, where that would make more than MAX_DECODE_BLOCKS workgroups, the multiple of 64
+//    that leaves the fullest compute unit the fewest keys (decode_split_len).  A row with several
 //    splits is finished by whichever of its blocks comes last (a ticket counter per row and kv
 //    head), which adds the partial results up in ascending split order: no second kernel, and the
 //    result does not depend on which block that was.  Splits and chunks are aligned to absolute
 //    positions.
+#include <map>
+#include <mutex>
+#include <tuple>
+
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -166,7 +171,7 @@ struct AttnArgs {
   float* part_o;   // [rows][nh][nsplit][HD]
   float* part_ml;  // [rows][nh][nsplit][2]
   int nsplit;
-  int split_len;   // positions per split, a multiple of 256
+  int split_len;   // positions per split, a multiple of 64
   int units;       // > 0: workgroups a kv head, which share the sequences' splits out among themselves
   int* tickets;    // [rows][nkv], zero between launches: how many splits of the row have finished
   // decode with the rotation and the cache write folded in (all null otherwise): the step's
@@ -1084,12 +1089,39 @@ bool lq_attention_mfma_accepts(int dtype, int nh, int nkv, int hd, int block_siz
   return true;
 }
 
-// Positions per block of a decoding launch.  It depends on the bound rounded up to 1024, so that
-// launches whose bounds differ less than that add up their sums in the same order.
+// Positions per block of a decoding launch: a multiple of 64 from 256 up, chosen so that the compute unit
+// with the most keys has as few as may be.  Workgroups go to the chip's dies in turn and within a die to its
+// compute units in turn, so with n workgroups the fullest unit has ceil(ceil(n / 8) / (units a die)) of them,
+// each with a split's keys; no more than MAX_DECODE_BLOCKS workgroups (two resident a unit), and of two
+// lengths that come to the same the shorter (more waves to hide each other's round trips).  It depends on the
+// bound rounded up to 1024, so that launches whose bounds differ less than that add up their sums in the same
+// order.
 static int decode_split_len(int rows, int nkv, int max_len) {
   const long long bound = (long long)lq_ceil_div(max_len, 1024) * 1024;
-  const long long per = ((long long)rows * nkv * bound + 256LL * MAX_DECODE_BLOCKS - 1) / (256LL * MAX_DECODE_BLOCKS);
-  return (int)(256 * (per > 1 ? per : 1));
+  // (asked for at every launch: the answers are kept)
+  static std::mutex guard;
+  static std::map<std::tuple<int, int, long long>, int> known;
+  const auto key = std::make_tuple(rows, nkv, bound);
+  {
+    std::lock_guard<std::mutex> lock(guard);
+    const auto it = known.find(key);
+    if (it != known.end()) return it->second;
+  }
+  const int per_die = lq_compute_units() / 8 > 0 ? lq_compute_units() / 8 : 1;
+  long long best = 0, best_cost = 0;
+  for (long long sl = 256; sl <= bound; sl += 64) {
+    const long long nsplit = (bound + sl - 1) / sl, blocks = (long long)rows * nkv * nsplit;
+    if (blocks > MAX_DECODE_BLOCKS && nsplit > 1) continue;
+    const long long on_fullest = ((blocks + 7) / 8 + per_die - 1) / per_die, cost = on_fullest * sl;
+    if (best == 0 || cost < best_cost) {
+      best = sl;
+      best_cost = cost;
+    }
+  }
+  const int answer = (int)(best > 0 ? best : bound);
+  std::lock_guard<std::mutex> lock(guard);
+  known[key] = answer;
+  return answer;
 }
 
 // Units a kv head for a decoding launch whose workgroups share the splits out themselves (0: the grid is
