@@ -783,7 +783,7 @@ __device__ inline int wave_prefix_sums(int v) {
 __device__ inline bool balanced_item(const AttnArgs& a, int u, DecodeItem& it) {
   const int lane = threadIdx.x & 63;
   const bool mine = lane < a.batch;
-  const int pl = mine ? a.row_pos[lane] : -1;  // lane l looks after sequence l (at most 32 of them)
+  const int pl = mine ? a.row_pos[lane] : -1;  // lane l looks after sequence l (at most 64 of them)
   const int sl = mine ? a.seq_slot[lane] : 0;
   const int total = __builtin_amdgcn_readlane(wave_prefix_sums(pl + 1), 63);
   // the smallest multiple of 256 with which the splits that hold keys are no more than the units; blocks of
@@ -1125,18 +1125,24 @@ static int decode_split_len(int rows, int nkv, int max_len) {
 }
 
 // Units a kv head for a decoding launch whose workgroups share the splits out themselves (0: the grid is
-// (sequence, kv head, split)): as many as keep the launch within MAX_DECODE_BLOCKS workgroups, no more than
-// the sequences have splits of 256 within their bound, and at least two a sequence.  Taken for 2 to 32
-// sequences without a window.
+// (sequence, kv head, split)): as many as keep the launch within MAX_DECODE_BLOCKS workgroups, or, where that
+// is less than two a sequence, LQ_UNITS_A_SEQUENCE a sequence (the workgroups beyond what a compute unit holds
+// wait their turn); no more than the sequences have splits of 256 within their bound, and at least two a
+// sequence, with which a split length that fits is sure to exist.  Taken for 2 to 64 sequences (a wave's
+// lanes) without a window.
+#ifndef LQ_UNITS_A_SEQUENCE
+#define LQ_UNITS_A_SEQUENCE 4
+#endif
 static int decode_units(int rows, int nkv, int max_len, int window) {
-  if (window > 0 || rows < 2 || rows > 32) return 0;
+  if (window > 0 || rows < 2 || rows > 64) return 0;
   const long long bound = (long long)lq_ceil_div(max_len, 1024) * 1024;
-  const long long by_cap = MAX_DECODE_BLOCKS / nkv, by_bound = (long long)rows * (bound / 256);
+  long long by_cap = MAX_DECODE_BLOCKS / nkv;
+  if (by_cap < 2 * rows) by_cap = (long long)LQ_UNITS_A_SEQUENCE * rows;
+  const long long by_bound = (long long)rows * (bound / 256);
   const long long units = by_cap < by_bound ? by_cap : by_bound;
-  if (units < 2 * rows) return 0;
-  // The split length is looked for upwards from (all keys) / (256 units) and found before twice that: with at
-  // least two units a sequence, splits of 2 (all keys) / units leave every sequence one to spare.  The kernel
-  // gives the search 1 024 steps.
+  if (units < 2 * rows || units > 65535) return 0;
+  // The kernel looks for the split length upwards from (all keys) / (256 units) and finds it before twice
+  // that; it gives the search 1 024 steps.
   if (rows * bound / (256 * units) > 512) return 0;
   return (int)units;
 }
@@ -1195,7 +1201,7 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
     a.split_len = decode_split_len(rows, nkv, max_len);
     a.nsplit = lq_ceil_div(max_len, a.split_len);
     LQ_REQUIRE(a.nsplit <= 65535, "attention: %d tokens are too many splits", max_len);
-    a.units = uneven && max_len > 256 ? decode_units(rows, nkv, max_len, window) : 0;
+    a.units = uneven ? decode_units(rows, nkv, max_len, window) : 0;  // (by the bound in 1 024s, as everything here)
     if (a.units > 0) {
       const long long need = (long long)a.units * nh * (hd + 2);
       LQ_REQUIRE(workspace != nullptr && workspace_floats >= need,

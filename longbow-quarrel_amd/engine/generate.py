@@ -317,7 +317,8 @@ class EngineBackend:
 
     def _decode_graph(self, slots: List[int], last_tokens: List[int], changed: bool) -> "_Launched":
         """The launched step whose tokens answer this call: the one queued ahead if it is the step asked
-        for (the same sequences, or some of them: a step's results do not depend on who else was in it),
+        for (the same sequences, or some of them: a step's results do not depend on who else was in it beyond
+        rounding, so a survivor's tokens can differ from a run without steps ahead where two candidates tie),
         else a step launched now.  Queues the step after it while the device still works on this one."""
         step, self.ahead = self.ahead, None
         if step is not None and not (set(slots) <= set(step.slots)):

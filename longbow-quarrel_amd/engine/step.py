@@ -31,9 +31,10 @@ from ..parts.base import BuildEnv, StepContext, Workspace
 def lengths_uneven(lengths: Sequence[int]) -> bool:
     """Whether the sequences of a decoding step differ so much in length (the longest at least half again
     as long as their mean) that the attention kernel does better sharing the keys out by the true lengths
-    than cutting every sequence as if it were the longest.  The one place where this is decided, for direct
-    and for captured steps alike, so that both sum in the same order."""
-    return len(lengths) >= 2 and 2 * len(lengths) * max(lengths) >= 3 * sum(lengths)
+    than cutting every sequence as if it were the longest; below 512 tokens there is nothing to share out.
+    The one place where this is decided, from the lengths alone, for direct and for captured steps alike,
+    so that both sum in the same order."""
+    return len(lengths) >= 2 and max(lengths) >= 512 and 2 * len(lengths) * max(lengths) >= 3 * sum(lengths)
 
 
 class SequenceTooLong(ValueError):

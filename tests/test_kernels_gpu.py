@@ -524,12 +524,15 @@ def test_rope_store_by_groups_of_eight_positions_writes_the_same_bits(kn, heads,
     (128, 4, 4, [600, 4700]),                                         # two sequences, no head shared
     (192, 6, 3, [2500, 10, 900]),                                     # (two waves a workgroup)
     (64, 8, 2, [260] * 3 + [3000] * 2 + [1] * 27),                    # 32 sequences, most of one token
+    (128, 8, 2, [4000, 3500] + [300 + 7 * i for i in range(38)] + [1, 2, 64, 65] * 6),  # 64 sequences: four units each
+    (64, 4, 4, [2500] + [90 + i for i in range(39)]),                 # 40 sequences
 ])
 def test_decode_attention_that_shares_its_keys_out_by_the_true_lengths(kn, head_dim, heads, kv_heads, lengths):
     """With the hint that the lengths are uneven the workgroups of a decoding launch number the splits that hold
     keys through (whole splits first, then every sequence's last) and each takes one, whatever sequence it belongs
     to: against the plain implementation, against the launch without the hint (the same sums in another order),
-    twice the same, the tickets back at zero; a far key that stands out is found in the long sequence."""
+    twice the same, the tickets back at zero; a far key that stands out is found in the long sequence.  Up to 64
+    sequences (a lane of a wave looks after each), from 33 on with four units a sequence."""
     n = len(lengths)
     got, want = run_attention(kn, None, lengths, [1] * n, heads, kv_heads, head_dim, torch.bfloat16, 41, decode=True,
                               uneven=True)
