@@ -136,3 +136,16 @@ def test_sampling_params_and_sequence_keys():
     keys = {sequence_key(s, i) for s in range(3) for i in range(50)}
     assert len(keys) == 150 and all(-(1 << 63) <= k < (1 << 63) for k in keys)
     assert sequence_key(1, 2) == sequence_key(1, 2)
+
+
+def test_when_a_step_calls_its_lengths_uneven():
+    """The hint to the attention kernel is a function of the lengths alone: the longest at least half again the
+    mean, two sequences or more, and something to share out (512 tokens)."""
+    from longbow_quarrel_amd.engine.step import lengths_uneven
+
+    assert lengths_uneven([3000, 1000]) and lengths_uneven([1401, 61, 26, 301]) and lengths_uneven([600, 200, 100])
+    assert not lengths_uneven([530] * 8) and not lengths_uneven([4000]) and not lengths_uneven([])
+    assert not lengths_uneven([1000, 985, 300])      # 1.31 times the mean
+    assert not lengths_uneven([500, 20, 30])         # nothing long enough to share out
+    assert lengths_uneven([1500, 1000, 500]) and not lengths_uneven([1499, 1000, 501])  # the bound itself: 1.5
+    assert lengths_uneven([5000] + [4000] * 63) is False and lengths_uneven([8000] + [100] * 63)
