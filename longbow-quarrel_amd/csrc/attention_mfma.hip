@@ -1092,8 +1092,10 @@ bool lq_attention_mfma_accepts(int dtype, int nh, int nkv, int hd, int block_siz
 // Positions per block of a decoding launch: a multiple of 64 from 256 up, chosen so that the compute unit
 // with the most keys has as few as may be.  Workgroups go to the chip's dies in turn and within a die to its
 // compute units in turn, so with n workgroups the fullest unit has ceil(ceil(n / 8) / (units a die)) of them,
-// each with a split's keys; no more than MAX_DECODE_BLOCKS workgroups (two resident a unit), and of two
-// lengths that come to the same the shorter (more waves to hide each other's round trips).  It depends on the
+// each with a split's keys; more than MAX_DECODE_BLOCKS workgroups (two resident a unit) only where that pays
+// for the waiting (33 to 63 long sequences, which one workgroup each would put two on some units and one on
+// others), and of two lengths that come to the same the shorter (more waves to hide each other's round
+// trips).  It depends on the
 // bound rounded up to 1024, so that launches whose bounds differ less than that add up their sums in the same
 // order.
 static int decode_split_len(int rows, int nkv, int max_len) {
@@ -1108,14 +1110,19 @@ static int decode_split_len(int rows, int nkv, int max_len) {
     if (it != known.end()) return it->second;
   }
   const int per_die = lq_compute_units() / 8 > 0 ? lq_compute_units() / 8 : 1;
-  long long best = 0, best_cost = 0;
+  long long best = 0, best_cost = 0, best_on = 0;
   for (long long sl = 256; sl <= bound; sl += 64) {
     const long long nsplit = (bound + sl - 1) / sl, blocks = (long long)rows * nkv * nsplit;
-    if (blocks > MAX_DECODE_BLOCKS && nsplit > 1) continue;
-    const long long on_fullest = ((blocks + 7) / 8 + per_die - 1) / per_die, cost = on_fullest * sl;
-    if (best == 0 || cost < best_cost) {
+    if (blocks > 4 * MAX_DECODE_BLOCKS && nsplit > 1) continue;
+    // (beyond the two workgroups that a compute unit holds at a time, each costs about 512 keys' worth of
+    // waiting for its turn and of round trips that nothing hides; where two lengths come to the same, the one
+    // with fewer workgroups a unit, and then the shorter)
+    const long long on_fullest = ((blocks + 7) / 8 + per_die - 1) / per_die;
+    const long long cost = on_fullest * sl + (on_fullest > 2 ? (on_fullest - 2) * 512 : 0);
+    if (best == 0 || cost < best_cost || (cost == best_cost && on_fullest < best_on)) {
       best = sl;
       best_cost = cost;
+      best_on = on_fullest;
     }
   }
   const int answer = (int)(best > 0 ? best : bound);
