@@ -14,7 +14,8 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
                       const int* block_table, int bt_stride, const void* kcache, const void* vcache,
                       float scale, int window, int decode, int max_len, float* workspace,
                       long long workspace_floats, int* tickets, long long tickets_n, const void* k_new,
-                      const void* v_new, int ldk, int ldv, const float* cs, int uneven, hipStream_t stream);
+                      const void* v_new, int ldk, int ldv, const float* cs, int uneven, int pieces,
+                      long long piece_stride, hipStream_t stream);
 
 // Floats of workspace lq_attention wants for this launch (0: none).
 extern "C" long long lq_attention_workspace(int dtype, int rows, int nh, int nkv, int hd, int block_size,
@@ -35,15 +36,17 @@ extern "C" int lq_attention_folds_rope(int dtype, int nh, int nkv, int hd, int b
 // counters that are zero between launches (a launch leaves them so): one for each row and kv head.
 // Launches that share them must not overlap.  `uneven` != 0 says that the sequences of a decoding launch
 // differ much in length: its workgroups then share the keys out among themselves by the true lengths
-// (the result is the same up to the order of its sums).
+// (the result is the same up to the order of its sums).  `pieces` > 1 (with cs only): q, k_new and v_new
+// are float32 partial sums of the projections, `pieces` of them `piece_stride` floats apart, and ldq, ldk
+// and ldv count floats; the launch adds them up in order and rounds the sums to the cache's dtype.
 extern "C" int lq_attention(const void* q, int ldq, void* out, int ldo, int dtype, int rows, int batch,
                             int nh, int nkv, int hd, const int* row_pos, const int* row_seq,
                             const int* seq_slot, const int* cu_rows, const int* block_table,
                             int bt_stride, const void* kcache, const void* vcache, int block_size,
                             float scale, int window, int decode, int max_len, float* workspace,
                             long long workspace_floats, int* tickets, long long tickets_n, const void* k_new,
-                            const void* v_new, int ldk, int ldv, const float* cs, int uneven,
-                            int force_generic, hipStream_t stream) {
+                            const void* v_new, int ldk, int ldv, const float* cs, int uneven, int pieces,
+                            long long piece_stride, int force_generic, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && batch > 0, "attention: rows %d and sequences %d must be positive", rows, batch);
   LQ_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "attention: %d heads over %d kv heads", nh, nkv);
   LQ_REQUIRE(hd > 0 && block_size > 0 && bt_stride > 0, "attention: bad sizes");
@@ -55,8 +58,8 @@ extern "C" int lq_attention(const void* q, int ldq, void* out, int ldo, int dtyp
     return lq_attention_mfma(q, ldq, out, ldo, rows, batch, nh, nkv, hd, row_pos, seq_slot, cu_rows,
                              block_table, bt_stride, kcache, vcache, scale, window, decode, max_len,
                              workspace, workspace_floats, tickets, tickets_n, k_new, v_new, ldk, ldv, cs, uneven,
-                             stream);
-  LQ_REQUIRE(cs == nullptr, "attention: the folded rotation was asked of a launch the matrix-core kernel does not take");
+                             pieces, piece_stride, stream);
+  LQ_REQUIRE(cs == nullptr && pieces <= 1, "attention: the folded rotation was asked of a launch the matrix-core kernel does not take");
   return lq_attention_generic(q, ldq, out, ldo, dtype, rows, nh, nkv, hd, row_pos, row_seq, seq_slot,
                               block_table, bt_stride, kcache, vcache, block_size, scale, window, stream);
 }

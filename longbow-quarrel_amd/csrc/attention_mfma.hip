@@ -180,6 +180,11 @@ struct AttnArgs {
   const bf16_t* v_new;
   int ldk, ldv;
   const float* cs;
+  // > 1 (folded launches only): q, k_new and v_new are float32, the partial sums that a product whose K was
+  // shared over blocks left, `pieces` of them `piece_stride` floats apart; ldq, ldk and ldv count floats.
+  // The kernel adds them up in order and rounds the sums as the whole product would have.
+  int pieces;
+  long long piece_stride;
 };
 
 // One chunk's operands as they come from memory: 16 bytes a lane for each K fragment and for each
@@ -815,7 +820,7 @@ __device__ inline bool balanced_item(const AttnArgs& a, int u, DecodeItem& it) {
   return true;
 }
 
-template <int HD, int NW>
+template <int HD, int NW, bool PIECES = false>
 __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int G = a.nh / a.nkv;
@@ -849,14 +854,69 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kerne
   const int h = kvh * G + min(c16, G - 1);
   const bool folded = HD % 64 == 0 && a.cs != nullptr;
   u32x4 qraw[HD / 32];
-  {
+  constexpr int KP = (HD / 2 + 63) / 64, VP = (HD + 63) / 64;
+  // (with pieces: the sums of this row's key pairs and value elements, lane i pair i and element i)
+  float pk0[KP], pk1[KP], pv[VP];
+  if constexpr (PIECES) {
+    // A few pieces are asked for together, everything a lane needs of them at once, and added in ascending
+    // order: one round trip for up to PC pieces.
+    constexpr int PC = HD <= 128 ? 4 : 2;
+    const float* qr = (const float*)a.q + (long long)r * a.ldq + h * HD + g * 8;
+    const float* kf = (const float*)a.k_new + (long long)r * a.ldk + kvh * HD;
+    const float* vf = (const float*)a.v_new + (long long)r * a.ldv + kvh * HD;
+    f32x4 sq[HD / 32][2];
+    for (int pc = 0; pc < a.pieces; pc += PC) {
+      f32x4 tq[PC][HD / 32][2];
+      float tk0[PC][KP], tk1[PC][KP], tv[PC][VP];
+#pragma unroll
+      for (int j = 0; j < PC; ++j) {
+        const long long at = (long long)min(pc + j, a.pieces - 1) * a.piece_stride;
+#pragma unroll
+        for (int kk = 0; kk < HD / 32; ++kk) {
+          tq[j][kk][0] = *(const f32x4*)(qr + at + kk * 32);
+          tq[j][kk][1] = *(const f32x4*)(qr + at + kk * 32 + 4);
+        }
+#pragma unroll
+        for (int e = 0; e < KP; ++e) {
+          const int i = min(lane + 64 * e, HD / 2 - 1);
+          tk0[j][e] = kf[at + i];
+          tk1[j][e] = kf[at + i + HD / 2];
+        }
+#pragma unroll
+        for (int e = 0; e < VP; ++e) tv[j][e] = vf[at + min(lane + 64 * e, HD - 1)];
+      }
+#pragma unroll
+      for (int j = 0; j < PC; ++j) {
+        if (pc + j >= a.pieces) continue;
+        const bool first = pc + j == 0;
+#pragma unroll
+        for (int kk = 0; kk < HD / 32; ++kk) {
+          sq[kk][0] = first ? tq[j][kk][0] : sq[kk][0] + tq[j][kk][0];
+          sq[kk][1] = first ? tq[j][kk][1] : sq[kk][1] + tq[j][kk][1];
+        }
+#pragma unroll
+        for (int e = 0; e < KP; ++e) {
+          pk0[e] = first ? tk0[j][e] : pk0[e] + tk0[j][e];
+          pk1[e] = first ? tk1[j][e] : pk1[e] + tk1[j][e];
+        }
+#pragma unroll
+        for (int e = 0; e < VP; ++e) pv[e] = first ? tv[j][e] : pv[e] + tv[j][e];
+      }
+    }
+#pragma unroll
+    for (int kk = 0; kk < HD / 32; ++kk) {
+      qraw[kk][0] = pack_bf16(sq[kk][0][0], sq[kk][0][1]);
+      qraw[kk][1] = pack_bf16(sq[kk][0][2], sq[kk][0][3]);
+      qraw[kk][2] = pack_bf16(sq[kk][1][0], sq[kk][1][1]);
+      qraw[kk][3] = pack_bf16(sq[kk][1][2], sq[kk][1][3]);
+    }
+  } else {
     const bf16_t* qr = a.q + (long long)r * a.ldq + h * HD + g * 8;
 #pragma unroll
     for (int kk = 0; kk < HD / 32; ++kk) qraw[kk] = *(const u32x4*)(qr + kk * 32);
   }
   // the row's own key and value (lane i: pair i of the key, elements d of the value), for the wave
   // that will turn out to write them
-  constexpr int KP = (HD / 2 + 63) / 64, VP = (HD + 63) / 64;
   float kx0[KP], kx1[KP], kc[KP], ks[KP];
   bf16_t vx[VP];
   if (folded) {
@@ -866,13 +926,21 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kerne
 #pragma unroll
     for (int j = 0; j < KP; ++j) {
       const int i = min(lane + 64 * j, HD / 2 - 1);
-      kx0[j] = bf16_to_f32(kr[i]);
-      kx1[j] = bf16_to_f32(kr[i + HD / 2]);
+      if constexpr (PIECES) {
+        kx0[j] = bf16_to_f32(f32_to_bf16(pk0[j]));
+        kx1[j] = bf16_to_f32(f32_to_bf16(pk1[j]));
+      } else {
+        kx0[j] = bf16_to_f32(kr[i]);
+        kx1[j] = bf16_to_f32(kr[i + HD / 2]);
+      }
       kc[j] = cs[2 * i];
       ks[j] = cs[2 * i + 1];
     }
 #pragma unroll
-    for (int j = 0; j < VP; ++j) vx[j] = vr[min(lane + 64 * j, HD - 1)];
+    for (int j = 0; j < VP; ++j) {
+      if constexpr (PIECES) vx[j] = f32_to_bf16(pv[j]);
+      else vx[j] = vr[min(lane + 64 * j, HD - 1)];
+    }
     // The rotation of this step's query, folded in.  Pair (i, i + HD/2): a lane's
     // fragment kk holds i = kk*32 + (lane/16)*8 + j and its fragment kk + HD/64 the partners.
 #pragma unroll
@@ -1069,7 +1137,12 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
   const int per_wave = (HD * G + 2 * G) * (int)sizeof(float);
   dim3 grid(a.batch, a.nkv, a.nsplit);
   if (a.units > 0) grid = dim3(a.nkv, a.units, 1);
-  if (4 * per_wave <= 48 * 1024)
+  if (a.pieces > 1) {
+    if (4 * per_wave <= 48 * 1024)
+      attn_heads_kernel<HD, 4, true><<<grid, 4 * 64, (size_t)4 * per_wave, stream>>>(a);
+    else
+      attn_heads_kernel<HD, 2, true><<<grid, 2 * 64, (size_t)2 * per_wave, stream>>>(a);
+  } else if (4 * per_wave <= 48 * 1024)
     attn_heads_kernel<HD, 4><<<grid, 4 * 64, (size_t)4 * per_wave, stream>>>(a);
   else
     attn_heads_kernel<HD, 2><<<grid, 2 * 64, (size_t)2 * per_wave, stream>>>(a);
@@ -1168,8 +1241,16 @@ int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int 
                       const int* block_table, int bt_stride, const void* kcache, const void* vcache,
                       float scale, int window, int decode, int max_len, float* workspace,
                       long long workspace_floats, int* tickets, long long tickets_n, const void* k_new,
-                      const void* v_new, int ldk, int ldv, const float* cs, int uneven, hipStream_t stream) {
+                      const void* v_new, int ldk, int ldv, const float* cs, int uneven, int pieces,
+                      long long piece_stride, hipStream_t stream) {
   AttnArgs a;
+  a.pieces = pieces;
+  a.piece_stride = piece_stride;
+  if (pieces > 1) {
+    LQ_REQUIRE(cs != nullptr, "attention: pieces of q, k and v are taken by the launch that rotates them only");
+    LQ_REQUIRE(pieces <= 64 && piece_stride > 0 && piece_stride % 4 == 0 && ldq % 4 == 0,
+               "attention: %d pieces %lld floats apart with rows of %d floats are not taken", pieces, piece_stride, ldq);
+  }
   a.q = (const bf16_t*)q;
   a.ldq = ldq;
   a.out = (bf16_t*)out;

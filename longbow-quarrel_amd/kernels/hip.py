@@ -20,7 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
-ABI_VERSION = 2  # lq_abi_version() of the library these wrappers were written for
+ABI_VERSION = 3  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -421,6 +421,12 @@ class HipKernels:
         return bool(self.lib.lq_attention_folds_rope(c_int(_DTYPE_CODE[dtype]), c_int(heads), c_int(kv_heads),
                                                      c_int(head_dim), c_int(block_size)))
 
+    @query
+    def attention_adds_pieces(self, dtype: torch.dtype, heads: int, kv_heads: int, head_dim: int, block_size: int) -> bool:
+        """Whether such a launch also takes q, k and v as the float32 pieces that `linear` leaves where it
+        shares K over blocks (`linear_pieces` > 1), and adds them up itself."""
+        return self.attention_folds_rope(dtype, heads, kv_heads, head_dim, block_size)
+
     def rope_table(self, freqs: torch.Tensor, row_pos: torch.Tensor, out: torch.Tensor) -> None:
         """out[r, i] = (cos, sin) of row_pos[r] * freqs[i]; float32 [rows, pairs, 2]."""
         self._dev(freqs, row_pos, out)
@@ -437,7 +443,7 @@ class HipKernels:
                   block_size: int, scale: float, window: int = 0, decode: bool = False, max_len: int = 0,
                   workspace: Optional[torch.Tensor] = None, k_new: Optional[torch.Tensor] = None,
                   v_new: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None,
-                  uneven: bool = False) -> None:
+                  uneven: bool = False, pieces: int = 1, piece_stride: int = 0) -> None:
         """Causal grouped-query attention of the step's rows over their slots' cached keys.
 
         `decode` promises one row per sequence; `max_len` is then an upper bound of the lengths
@@ -446,7 +452,9 @@ class HipKernels:
         context knows): the launch then shares the keys out over its workgroups by the true lengths.
         With `cos_sin` (a `rope_table` of this step; only where `attention_folds_rope` says so) q, k_new
         and v_new are the unrotated projections: the launch rotates q and k and writes k and v into
-        the cache itself."""
+        the cache itself.  With `pieces` > 1 (such a launch only, where `attention_adds_pieces` says so)
+        q, k_new and v_new are float32 views into the first of that many partial sums of the projection,
+        `piece_stride` elements apart (what `linear` leaves in a 3-D out): the launch adds them up."""
         self._dev(q, out, row_pos, row_seq, seq_slot, cu_rows, block_table, kcache, vcache, workspace)
         rows = q.shape[0]
         batch = seq_slot.numel()
@@ -455,8 +463,11 @@ class HipKernels:
         self._i32(cu_rows, "cu_rows", batch + 1)
         if out.shape[0] != rows or out.shape[1] < heads * head_dim or q.shape[1] < heads * head_dim:
             raise KernelLibraryError("attention: q / out do not match rows x heads*head_dim")
-        if q.dtype != out.dtype or kcache.dtype != q.dtype or vcache.dtype != q.dtype:
-            raise KernelLibraryError("attention: q, out and the caches must share one dtype")
+        taken = torch.float32 if pieces > 1 else out.dtype
+        if q.dtype != taken or kcache.dtype != out.dtype or vcache.dtype != out.dtype:
+            raise KernelLibraryError("attention: q, out and the caches must share one dtype (pieces of q are float32)")
+        if pieces > 1 and (cos_sin is None or piece_stride <= 0):
+            raise KernelLibraryError("attention: pieces of q, k and v go with the folded rotation only")
         nb = kcache.shape[0]
         if tuple(kcache.shape) != (nb, kv_heads, block_size, head_dim) or \
                 tuple(vcache.shape) != (nb, kv_heads, head_dim, block_size) or \
@@ -484,13 +495,14 @@ class HipKernels:
             ldk, ldv = self._rows2d(k_new, "k_new"), self._rows2d(v_new, "v_new")
         rc = self.lib.lq_attention(
             _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")),
-            c_int(_code(q)), c_int(rows), c_int(batch), c_int(heads), c_int(kv_heads), c_int(head_dim),
+            c_int(_code(out)), c_int(rows), c_int(batch), c_int(heads), c_int(kv_heads), c_int(head_dim),
             _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(cu_rows), _ptr(block_table),
             c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
             c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
             c_longlong(ws_n), _ptr(self._tickets), c_longlong(self._tickets.numel()), _ptr(k_new if cos_sin is not None else None),
             _ptr(v_new if cos_sin is not None else None), c_int(ldk), c_int(ldv), _ptr(cos_sin),
-            c_int(1 if uneven and decode else 0), c_int(1 if self.force_generic else 0), self.stream)
+            c_int(1 if uneven and decode else 0), c_int(pieces), c_longlong(piece_stride),
+            c_int(1 if self.force_generic else 0), self.stream)
         if rc != 0:
             # a launch that did not run whole may have left tickets behind, and a later launch that found
             # them non-zero would never recognise its last workgroup: clear them (a fill kernel) before

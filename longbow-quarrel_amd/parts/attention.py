@@ -72,28 +72,42 @@ class GQAttention(Mixer):
             raise RuntimeError("attention needs a key/value cache")
         kn = ctx.kernels
         rows = h.shape[0]
-        qkv = ctx.ws.alloc((rows, self.q_width + 2 * self.kv_width), ctx.dtype)
-        if not project_normed(kn, ctx, h, self.w_qkv, qkv):
-            if isinstance(h, NormedRows):
-                h = h.tensor(ctx)
-            project(kn, ctx, h, self.w_qkv, qkv)
-        q = qkv[:, : self.q_width]
-        k = qkv[:, self.q_width : self.q_width + self.kv_width]
-        v = qkv[:, self.q_width + self.kv_width :]
         freqs = self.position.rotary_frequencies
+        shape = (ctx.dtype, self.heads, self.kv_heads, self.head_dim, cache.block_size)
+        # a decoding step can leave the rotation and the cache write to the attention kernel itself
+        folded = (ctx.decode and cache.write and freqs is not None and hasattr(self.position, "cos_sin")
+                  and getattr(kn, "attention_folds_rope", lambda *a: False)(*shape))
+        width = self.q_width + 2 * self.kv_width
+        # ... and then also the adding up of q, k and v, where the product would rather share K over blocks
+        # (a few dozen rows: its columns alone are too few for the chip)
+        pieces = 1
+        if (folded and not isinstance(h, NormedRows) and self.w_qkv.dtype == h.dtype
+                and getattr(kn, "attention_adds_pieces", lambda *a: False)(*shape)):
+            pieces = kn.linear_pieces(h.dtype, rows, width, self.width)
+        if pieces > 1:
+            qkv = ctx.ws.alloc((pieces, rows, width), torch.float32)
+            project(kn, ctx, h, self.w_qkv, qkv)
+            first, stride = qkv[0], qkv.stride(0)
+        else:
+            qkv = first = ctx.ws.alloc((rows, width), ctx.dtype)
+            stride = 0
+            if not project_normed(kn, ctx, h, self.w_qkv, qkv):
+                if isinstance(h, NormedRows):
+                    h = h.tensor(ctx)
+                project(kn, ctx, h, self.w_qkv, qkv)
+        q = first[:, : self.q_width]
+        k = first[:, self.q_width : self.q_width + self.kv_width]
+        v = first[:, self.q_width + self.kv_width :]
         att = ctx.ws.alloc((rows, self.q_width), ctx.dtype)
         need = kn.attention_workspace(ctx.dtype, rows, self.heads, self.kv_heads, self.head_dim,
                                       cache.block_size, ctx.decode, ctx.max_len)
         scratch = ctx.ws.alloc((need,), torch.float32) if need else None
-        # a decoding step can leave the rotation and the cache write to the attention kernel itself
-        folded = (ctx.decode and cache.write and freqs is not None and hasattr(self.position, "cos_sin")
-                  and getattr(kn, "attention_folds_rope", lambda *a: False)(
-                      ctx.dtype, self.heads, self.kv_heads, self.head_dim, cache.block_size))
         if folded:
+            more = dict(pieces=pieces, piece_stride=stride) if pieces > 1 else {}
             kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
                          ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
                          self.scale, self.window, decode=True, max_len=ctx.max_len, workspace=scratch,
-                         k_new=k, v_new=v, cos_sin=self.position.cos_sin(ctx), uneven=ctx.uneven)
+                         k_new=k, v_new=v, cos_sin=self.position.cos_sin(ctx), uneven=ctx.uneven, **more)
         else:
             if freqs is None:
                 self.position.apply(q, k, ctx)

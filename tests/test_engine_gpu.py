@@ -355,9 +355,22 @@ def test_decoding_batches_that_shrink_from_40_rows_to_one(tmp_path_factory):
     """40 sequences that end one after the other: decoding steps of 40 down to 1 row take the pipelined
     64-row tiles (above 32 rows), then the matrix-vector kernels with two and one row tile (K shared
     between blocks, the pieces added by the norms; below 17 rows the norms folded into the products),
-    against the plain implementation."""
-    folder = write_folder(tmp_path_factory.mktemp("wide64"), WIDE, seed=4, std=0.03)
+    against the plain implementation.  From 17 rows on q, k and v leave their product in pieces too, which
+    the decoding attention adds up (a width that is a multiple of 256, so that K can be shared, and no more
+    than 16 heads a kv head, which is what the matrix-core decoding attention takes)."""
+    wide = dict(WIDE, hidden_size=2304, num_attention_heads=18, num_key_value_heads=2)
+    folder = write_folder(tmp_path_factory.mktemp("wide64"), wide, seed=4, std=0.03)
     eng = lq.load_engine(folder, dtype="bfloat16", max_tokens=64 * 48)
+    kn = eng.kernels
+    in_pieces = set()
+    attention = kn.attention
+
+    def watched(q, *a, **k):
+        if k.get("pieces", 1) > 1:
+            in_pieces.add(q.shape[0])
+        return attention(q, *a, **k)
+
+    kn.attention = watched
     c, tensors = read_folder(folder)
     ref = plain.PlainLlama(c, tensors)
     reqs = [random_tokens(4 + (i * 7) % 23, WIDE["vocab_size"], 500 + i) for i in range(40)]
@@ -376,9 +389,11 @@ def test_decoding_batches_that_shrink_from_40_rows_to_one(tmp_path_factory):
         for j, i in enumerate(live):
             out[i].append(got[j : j + 1])
         pos += 1
+    kn.attention = attention
     for i, w in enumerate(want):
         assert rel_err(torch.cat(out[i]), w) < TOL_BF16, i
     assert any(r > 32 for r in rows_seen) and any(16 < r <= 32 for r in rows_seen) and any(r <= 16 for r in rows_seen)
+    assert any(r > 32 for r in in_pieces) and any(16 < r <= 32 for r in in_pieces) and not any(r <= 16 for r in in_pieces)
 
 
 LONG = {

@@ -616,3 +616,52 @@ def test_decode_attention_with_rotation_and_cache_write_folded_in(kn, heads, kv_
     assert torch.equal(kc, kc2) and torch.equal(vc, vc2)  # the same rows of the cache were written, with the same bits
     assert rel_err(out_b, out_a.double().cpu()) < 4e-3
 
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,pieces", [(32, 8, 128, 4), (4, 2, 64, 2), (16, 1, 64, 7), (6, 3, 192, 3)])
+@pytest.mark.parametrize("uneven", [False, True])
+def test_decode_attention_that_adds_up_the_pieces_of_its_projections(kn, heads, kv_heads, head_dim, pieces, uneven):
+    """The folded launch given q, k and v as float32 partial sums (what a product leaves that shares K over
+    blocks) against the same launch given their sums rounded to bfloat16: the same bits, in the output and in
+    the cache."""
+    from longbow_quarrel_amd.kernels.hip import KernelLibraryError
+    dtype = torch.bfloat16
+    lengths = [700, 64, 257, 1, 1300, 2, 900]
+    assert kn.attention_adds_pieces(dtype, heads, kv_heads, head_dim, BS)
+    kc, vc, table, slots, dense = paged_cache(lengths, kv_heads, head_dim, dtype, 61)
+    kc2, vc2 = kc.clone(), vc.clone()
+    rows = len(lengths)
+    width = (heads + 2 * kv_heads) * head_dim
+    parts = rnd((pieces, rows, width), 62, torch.float32)
+    whole = parts[0].clone()
+    for i in range(1, pieces):  # in this order, as the launch adds them
+        whole = whole + parts[i]
+    whole = whole.to(dtype)
+    pos = [n - 1 for n in lengths]
+    freqs = plain.rope_frequencies(head_dim, 500000.0).to(DEV)
+    cu = list(range(rows + 1))
+    scale = 1.0 / math.sqrt(head_dim)
+    need = kn.attention_workspace(dtype, rows, heads, kv_heads, head_dim, BS, True, max(lengths))
+    ws = torch.empty(max(need, 1), dtype=torch.float32, device=DEV)
+    cs = torch.empty((rows, head_dim // 2, 2), dtype=torch.float32, device=DEV)
+    kn.rope_table(freqs, i32(pos), cs)
+
+    def views(t):
+        return t[:, : heads * head_dim], t[:, heads * head_dim : (heads + kv_heads) * head_dim], t[:, (heads + kv_heads) * head_dim :]
+
+    outs = []
+    for src, k_cache, v_cache, more in ((whole, kc, vc, {}),
+                                        (parts[0], kc2, vc2, dict(pieces=pieces, piece_stride=parts.stride(0)))):
+        q, k, v = views(src)
+        out = torch.empty((rows, heads * head_dim), dtype=dtype, device=DEV)
+        kn.attention(q, out, heads, kv_heads, head_dim, i32(pos), i32(range(rows)), i32(slots), i32(cu), table,
+                     k_cache, v_cache, BS, scale, 0, decode=True, max_len=max(lengths), workspace=ws, k_new=k,
+                     v_new=v, cos_sin=cs, uneven=uneven, **more)
+        outs.append(out)
+    assert torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    assert torch.equal(outs[0], outs[1])
+    with pytest.raises(KernelLibraryError):  # pieces without the folded rotation: refused
+        q, k, v = views(parts[0])
+        kn.attention(q, outs[1], heads, kv_heads, head_dim, i32(pos), i32(range(rows)), i32(slots), i32(cu), table,
+                     kc2, vc2, BS, scale, 0, decode=True, max_len=max(lengths), workspace=ws, pieces=pieces,
+                     piece_stride=parts.stride(0))
+
