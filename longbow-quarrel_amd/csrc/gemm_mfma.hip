@@ -917,11 +917,30 @@ inline bool mid_rows(int M, int N, int K) {
   return M > 32 && M <= 256 && K % 64 == 0 && K >= 512 && N >= 8 * lq_compute_units();
 }
 
-int mid_splits(int M, int N, int K) {
-  const int tiles = lq_ceil_div(N, 128), want = 3 * lq_compute_units() / 4;
+inline int mid_splits_for(int tiles, int K) {
+  const int want = 3 * lq_compute_units() / 4;
   int splits = 1;
   while (splits < 16 && tiles * splits < want && K % (128 * splits) == 0 && K / (2 * splits) >= 512) splits *= 2;
   return splits;
+}
+
+// Up to 64 rows, a product in pieces may take 64-column tiles (four waves) instead of 128-column ones (eight):
+// as many blocks with half as many pieces for the consumer to add.  They are taken where they give more blocks,
+// or as many when these fill every compute unit (then the chip's memory bounds the launch, and fewer pieces are
+// what is left to gain: 8B shape at 64 rows, the norm after o and down 7.8 -> 6.9 us); where blocks are fewer
+// than compute units a block's bytes in flight bound it, and the wide tile has twice as many (q, k and v at 64
+// rows: 13.2 against 16.0 us).
+inline bool mid_narrow(int M, int N, int K) {
+  if (M > 64) return false;
+  const int cus = lq_compute_units();
+  const int wide = lq_ceil_div(N, 128) * mid_splits_for(lq_ceil_div(N, 128), K);
+  const int narrow = lq_ceil_div(N, 64) * mid_splits_for(lq_ceil_div(N, 64), K);
+  if (mid_splits_for(lq_ceil_div(N, 64), K) == 1) return false;  // whole: the 128-column tile or its siblings below
+  return (narrow < cus ? narrow : cus) > (wide < cus ? wide : cus) || (narrow >= cus && wide >= cus);
+}
+
+int mid_splits(int M, int N, int K) {
+  return mid_splits_for(lq_ceil_div(N, mid_narrow(M, N, K) ? 64 : 128), K);
 }
 
 template <int EPI, typename TO>
@@ -941,6 +960,9 @@ int launch_mid(const void* x, const void* w, void* out, int M, int N, int K, int
       return launch_pipelined<4, 2, 2, 1, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
     }
   }
+  if constexpr (EPI == EPI_NONE)
+    if (splits > 1 && mid_narrow(M, N, K))
+      return launch_pipelined<2, 2, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
   if (M <= 64)
     return launch_pipelined<2, 4, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
   if (M <= 128)
