@@ -138,7 +138,7 @@ def test_linear_bfloat16_matrix_cores(kn, out_dtype, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(64, 4096, 4096), (17, 4096, 14336), (40, 2560, 2056), (33, 6144, 4096),
                                    (300, 4096, 4096), (2048, 4096, 14336), (65, 1000, 2048), (130, 4096, 14336),
-                                   (256, 2100, 1024)])
+                                   (256, 2100, 1024), (50, 2100, 1024)])  # (the last: 64-column tiles with an edge)
 def test_linear_in_pieces_and_their_consumers(kn, m, n, k):
     """Few columns and several row tiles: K is shared out over blocks and the product comes as
     pieces; the norm, the add and the row gather that take such a delta add the pieces up."""
