@@ -315,6 +315,8 @@ __global__ void gather_rows_kernel(const float* __restrict__ x, const TD* __rest
                                    int D) {
   const long long src = (long long)rows[blockIdx.x] * D;
   const long long dst = (long long)blockIdx.x * D;
+  // (a launch of a few rows is bound by the latency of its loads: those of four turns are asked for together)
+#pragma unroll 4
   for (int j = threadIdx.x; j < D; j += blockDim.x) {
     float v = x[src + j];
     if (HAS_DELTA) {
