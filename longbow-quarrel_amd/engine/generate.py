@@ -92,20 +92,25 @@ class GenerationLoop:
         self.max_batch = max_batch
 
     def _next_batch(self, pending: List[int], prompts: Sequence[Sequence[int]], limit: Sequence[int]) -> List[int]:
-        """The longest prefix of the pending requests that fits the batch size and the cache."""
+        """The longest prefix of the pending requests that fits the batch size and the cache.  A request
+        caches its prompt and every token it is given but the last, which is sampled and never fed back."""
         budget = self.backend.free_blocks()
         chosen: List[int] = []
         for r in pending:
-            need = self.backend.blocks_needed(len(prompts[r]) + limit[r])
+            need = self.backend.blocks_needed(self._cached_tokens(prompts[r], limit[r]))
             if len(chosen) >= self.max_batch or need > budget:
                 break
             chosen.append(r)
             budget -= need
         if not chosen:
             r = pending[0]
-            raise CacheFull(
-                f"request {r} needs room for {len(prompts[r]) + limit[r]} tokens, more than the cache can hold")
+            raise CacheFull(f"request {r} needs room for {self._cached_tokens(prompts[r], limit[r])} tokens, "
+                            "more than the cache can hold")
         return chosen
+
+    @staticmethod
+    def _cached_tokens(prompt: Sequence[int], limit: int) -> int:
+        return len(prompt) + max(limit, 1) - 1
 
     def _token_limits(self, prompts: Sequence[Sequence[int]], max_new_tokens: int) -> List[int]:
         """How many tokens each request may get: `max_new_tokens`, or fewer where the sequence would

@@ -295,6 +295,21 @@ def test_generation_stops_where_a_sequence_may_not_grow_further(tmp_path):
     assert eng.cache.slots.taken_count == 0
 
 
+def test_the_whole_cache_is_reachable_when_pool_and_sequence_bound_are_one_figure(tmp_path):
+    """The cache's pool and the bound of a sequence are the same 128 tokens (what the facade, the replay tool
+    and the command line with one prompt set up): a prompt of 10 tokens gets 119 tokens, the last of them
+    sampled from position 127 (the reference accepts positions below its cache size:
+    internal/engine/kv_cache.go:121-124), and a larger request is clipped there, not refused."""
+    eng, ref = make(tmp_path, TINY_A, max_tokens=128, max_sequence_tokens=128)
+    prompt = random_tokens(10, 256, 3)
+    res = lq.generate(eng, [prompt], 119, stop_ids=[], use_graphs=False)
+    assert [len(t) for t in res.tokens] == [119] and res.finish == ["length"]
+    for n in (120, 500):
+        more = lq.generate(eng, [prompt], n, stop_ids=[], use_graphs=False)
+        assert more.tokens == res.tokens and more.finish == ["length"], n
+    assert eng.cache.slots.taken_count == 0 and eng.cache.free_blocks() == 2
+
+
 def test_non_finite_logits_are_reported_not_sampled(tmp_path):
     """A NaN or an infinity among a row's logits stops generation with an error that names the request
     (the reference would go on from the first finite index: internal/engine/sampler.go:72-75, 107-123)."""

@@ -105,6 +105,16 @@ def test_batches_are_cut_by_what_the_cache_can_hold():
         GenerationLoop(ScriptedBackend(blocks=2), max_batch=8).run([[1] * 200], 10)
 
 
+def test_the_last_sampled_token_takes_no_room_in_the_cache():
+    """A request caches its prompt and all its tokens but the last (sampled, never fed back): a prompt of
+    10 tokens with 119 to come fills exactly two blocks of 64, and one with 120 to come needs a third."""
+    be = ScriptedBackend(blocks=2)
+    res = GenerationLoop(be, max_batch=8).run([[1] * 10], 119, stop_ids=[])
+    assert len(res.tokens[0]) == 119
+    with pytest.raises(CacheFull, match="129 tokens"):
+        GenerationLoop(ScriptedBackend(blocks=2), max_batch=8).run([[1] * 10], 120, stop_ids=[])
+
+
 def test_degenerate_requests():
     be = ScriptedBackend()
     assert GenerationLoop(be).run([], 5).tokens == []
