@@ -8,7 +8,13 @@ exactly K timed ones (a step = one token for every sequence of the batch: model,
 greedy sampling on the device and state upkeep, replayed as a HIP graph, tokens read
 back by the host every step as generation does).  `value` is decoded tokens a
 second.  The same line carries a 2,048-token prefill, the decode step's HBM
-roofline, and decode at batch 1 and 64.  One JSON line on stdout.
+roofline, and as `points` decode at batch 1 and 64, prefills of 512 and 8,192 tokens
+(tokens a second) and decode at batch 8 from prompts of 8,192 and 32,768 tokens (the
+pool of the 64 x 8,192-token cache holds them; only the bound of one sequence is raised
+for these).  One JSON line on stdout.
+
+`--dtype float32` runs the true 32-bit path (float32 weights, cache and activations; peaks:
+157.3 TFLOP/s, the same 8 TB/s); with the 8B shape that is for a few layers (`--layers 4`).
 
 `--shape 1b`: the Llama 3.2 1B layer sizes, 16 prompts of 64 to 4,096 tokens (uniform, from a
 seed) and then K decoding steps, all of it through the generation loop (`GenerationLoop.run`:
@@ -30,6 +36,7 @@ if ROOT not in sys.path:
 
 HBM_GBPS = 8000.0  # MI355X published peak
 BF16_TFLOPS = 2500.0  # dense MFMA bf16
+FP32_TFLOPS = 157.3  # dense MFMA fp32
 
 CONFIG_8B = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "intermediate_size": 14336,
@@ -49,17 +56,17 @@ CONFIG_70B = dict(CONFIG_8B, hidden_size=8192, intermediate_size=28672, num_hidd
 SHAPES = {"8b": CONFIG_8B, "1b": CONFIG_1B, "70b": CONFIG_70B}
 
 
-def weight_bytes_per_step(c) -> float:
-    """Every weight a decode step uses, once: the layers' matrices and norms, the final norm and the head
-    (of the embedding table only the batch's rows are read)."""
+def weight_bytes_per_step(c, element: int = 2) -> float:
+    """Every weight a decode step uses, once: the layers' matrices (`element` bytes an entry) and norms
+    (always float32), the final norm and the head (of the embedding table only the batch's rows are read)."""
     d, i, hd = c.hidden_size, c.intermediate_size, c.head_dim
     nh, nkv = c.num_attention_heads, c.num_key_value_heads
-    per_layer = 2 * (d * (nh + 2 * nkv) * hd + nh * hd * d + 3 * d * i) + 4 * 2 * d
-    return c.num_hidden_layers * per_layer + 2 * c.vocab_size * d + 4 * d
+    per_layer = element * (d * (nh + 2 * nkv) * hd + nh * hd * d + 3 * d * i) + 4 * 2 * d
+    return c.num_hidden_layers * per_layer + element * c.vocab_size * d + 4 * d
 
 
-def kv_bytes_per_token(c) -> float:
-    return 2 * c.num_key_value_heads * c.head_dim * 2 * c.num_hidden_layers
+def kv_bytes_per_token(c, element: int = 2) -> float:
+    return 2 * c.num_key_value_heads * c.head_dim * element * c.num_hidden_layers
 
 
 def prefill_flops(c, t: int) -> float:
@@ -87,6 +94,8 @@ def main() -> int:
     ap.add_argument("--prefill-only", action="store_true", help="run the prefill alone, twice (for profiling)")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="prompt length of --prefill-only (the reported prefill is always of 2,048 tokens)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
+                    help="float32: the true 32-bit path (use --layers with the larger shapes)")
     ap.add_argument("--context", type=int, default=0,
                     help="tokens a sequence may hold (default: the shape's 8192); for decoding over longer prompts")
     args = ap.parse_args()
@@ -114,7 +123,9 @@ def main() -> int:
     slot_len = cfg["max_position_embeddings"]
     max_batch = 64 if (args.shape == "8b" and not (args.no_points or args.prefill_only)) else args.batch
     t0 = time.time()
-    engine = lq.random_engine(config, seed=0, dtype="bfloat16", max_tokens=max_batch * slot_len, max_slots=max_batch)
+    element = 2 if args.dtype == "bfloat16" else 4
+    peak_tflops = BF16_TFLOPS if args.dtype == "bfloat16" else FP32_TFLOPS
+    engine = lq.random_engine(config, seed=0, dtype=args.dtype, max_tokens=max_batch * slot_len, max_slots=max_batch)
     torch.cuda.synchronize()
     print(f"[bench] model and cache ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
     gen = torch.Generator().manual_seed(1234)
@@ -124,6 +135,9 @@ def main() -> int:
 
     def decode_run(batch: int, prompt_len: int, steps: int, warmup: int):
         """tokens a second, ms a step, mean context during the timed steps"""
+        # (a point over a longer context than the configuration's: the pool holds it, the bound of one
+        # sequence is raised for it)
+        engine.max_sequence_tokens = max(engine.max_sequence_tokens, prompt_len + steps + warmup + 2)
         backend = EngineBackend(engine, lq.SamplingParams(temperature=0.0), use_graphs=True)
         slots = [backend.new_sequence(r, [0]) for r in range(batch)]
         lens = [prompt_len] * batch
@@ -178,7 +192,7 @@ def main() -> int:
             engine.release(slot)
         dt = sorted(times)[1]
         return {"value": round(t_tokens / dt, 1), "tokens": t_tokens, "ms": round(dt * 1e3, 3),
-                "frac": round(prefill_flops(config, t_tokens) / dt / (BF16_TFLOPS * 1e12), 4)}
+                "frac": round(prefill_flops(config, t_tokens) / dt / (peak_tflops * 1e12), 4)}
 
     prefill = None
     points = {}
@@ -201,10 +215,10 @@ def main() -> int:
         flops = sum(prefill_flops(config, n) for n in lens)
         prefill = {"value": round(n_prompt / res.prefill_seconds, 1), "tokens": n_prompt,
                    "ms": round(res.prefill_seconds * 1e3, 3),
-                   "frac": round(flops / res.prefill_seconds / (BF16_TFLOPS * 1e12), 4)}
+                   "frac": round(flops / res.prefill_seconds / (peak_tflops * 1e12), 4)}
     else:
         value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
-    step_bytes = weight_bytes_per_step(config) + args.batch * ctx_mean * kv_bytes_per_token(config)
+    step_bytes = weight_bytes_per_step(config, element) + args.batch * ctx_mean * kv_bytes_per_token(config, element)
     achieved = step_bytes / (ms_step * 1e-3) / 1e9
     print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
 
@@ -216,15 +230,23 @@ def main() -> int:
         if args.shape == "8b":
             v64, _, _ = decode_run(64, args.prompt_len, max(16, args.steps // 4), max(4, args.warmup // 2))
             points["decode_b64"] = round(v64, 1)
+        if args.shape == "8b" and args.dtype == "bfloat16" and not args.layers and not args.context:
+            # further prompt lengths and contexts, so that whoever runs the default line times them too
+            for n in (512, 8192):
+                points[f"prefill_{n}"] = prefill_point(n)["value"]
+            for ctx in (8192, 32768):
+                if args.batch * (ctx + 64) <= max_batch * slot_len:
+                    v, _, _ = decode_run(args.batch, ctx, max(8, args.steps // 4), max(2, args.warmup // 4))
+                    points[f"decode_b{args.batch}_ctx{ctx}"] = round(v, 1)
         print(f"[bench] points: {points}", file=sys.stderr, flush=True)
 
     line = {
-        "metric": f"decode tok/s (Llama-3 {args.shape.upper()} shape, bf16, batch {args.batch}, " + (
+        "metric": f"decode tok/s (Llama-3 {args.shape.upper()} shape, {'bf16' if element == 2 else 'fp32'}, batch {args.batch}, " + (
             f"prompts of {args.prompt_len} to {args.prompt_len_max} tokens)" if args.prompt_len_max > args.prompt_len
             else f"{args.prompt_len}-token prompts)"),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic: random weights N(0, 0.02) from a seed, uniform random token ids",
+        "dtype": "bf16" if element == 2 else "fp32", "data": "synthetic: random weights N(0, 0.02) from a seed, uniform random token ids",
         "config": {
             "model": f"llama3-{args.shape}-shape", "layers": config.num_hidden_layers, "layers_full": full_layers,
             "hidden": config.hidden_size, "heads": config.num_attention_heads,

@@ -61,6 +61,9 @@ class CacheGroup:
     def ensure(self, slot: int, new_len: int) -> None:
         """Room for positions < new_len (the manager has checked `blocks_missing` against `free_blocks`)."""
 
+    def reserved(self) -> None:
+        """Every `ensure` of one `CacheManager.reserve` has been made."""
+
     def trim(self, slot: int, length: int) -> None:
         """The slot holds `length` tokens now; what no later token can reach may go back."""
 
@@ -88,7 +91,14 @@ class KVGroup(CacheGroup):
         self.k = torch.zeros(shape_k, dtype=dtype, device=device)
         self.v = torch.zeros(shape_v, dtype=dtype, device=device)
         self.table_width = max(1, self.n_blocks)
-        self.table_host = torch.zeros((self.max_slots, self.table_width), dtype=torch.int32)
+        # The host's copy is pinned: new entries go up without a wait for the device, so a step queued ahead
+        # stays queued when a sequence crosses a block's edge.  A row is only ever appended to while its
+        # sequence lives; before a row is written from its start again (the slot has a new sequence) the
+        # uploads asked for so far are waited for (`_uploaded`), since they read this memory when they run.
+        self.table_host = torch.zeros((self.max_slots, self.table_width), dtype=torch.int32,
+                                      pin_memory=device.type == "cuda")
+        self._uploaded: Optional["torch.cuda.Event"] = None
+        self._uploads_pending = False
         self.table_dev = torch.zeros((self.max_slots, self.table_width), dtype=torch.int32, device=device)
         # per slot: physical block of each logical block (None once trimmed away)
         self.owned: List[List[Optional[int]]] = [[] for _ in range(self.max_slots)]
@@ -120,8 +130,18 @@ class KVGroup(CacheGroup):
         if want > self.table_width:
             raise CacheFull(f"a sequence of {new_len} tokens needs {want} blocks, the table holds {self.table_width}")
         owned.extend(self.blocks.take_many(want - first))
+        if first == 0 and self._uploaded is not None:
+            self._uploaded.synchronize()
+            self._uploaded = None
         self.table_host[slot, first:want] = torch.tensor(owned[first:want], dtype=torch.int32)
-        self.table_dev[slot, first:want].copy_(self.table_host[slot, first:want])
+        self.table_dev[slot, first:want].copy_(self.table_host[slot, first:want], non_blocking=True)
+        self._uploads_pending = True
+
+    def reserved(self) -> None:
+        if self._uploads_pending and self.table_dev.is_cuda:
+            self._uploaded = torch.cuda.Event()
+            self._uploaded.record()
+        self._uploads_pending = False
 
     def trim(self, slot: int, length: int) -> None:
         """A windowed group gives back the blocks no later query can reach."""
@@ -223,6 +243,7 @@ class CacheManager:
         for g in self.groups:
             for slot, n in growth.items():
                 g.ensure(slot, self.lengths[slot] + n)
+            g.reserved()
 
     def advance(self, growth: Mapping[int, int]) -> None:
         for slot, n in growth.items():

@@ -7,7 +7,9 @@ names and meanings where it has them.
 `-model` is a folder with config.json and model.safetensors (env QUARREL_MODEL if the
 option is absent, as generate_text does).  `-prompt` is text when the folder has a
 tokenizer.json, else token ids separated by blanks or commas; several prompts are
-separated by `|` and run as one batch.  The beginning-of-sequence id of the
+separated by `|` and run as one batch; `-prompt-file` reads them from a file instead, one prompt a
+line; `-prompt-ids` always takes token ids.  `-stop-id` (repeatable) names ids that end a sequence beside
+the configuration's own.  The beginning-of-sequence id of the
 configuration is put in front of text prompts (the reference prepends id 1,
 cmd/quarrel/main_metal.go:113-114).
 """
@@ -25,7 +27,14 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("-model", "--model", default=os.environ.get("QUARREL_MODEL", ""),
                     help="folder with config.json and model.safetensors (or env QUARREL_MODEL)")
     ap.add_argument("-prompt", "--prompt", default="1", help="text, or token ids; '|' separates several prompts")
-    ap.add_argument("-n", "--n", "-len", "--len", dest="n", type=int, default=20, help="number of tokens to generate")
+    ap.add_argument("-prompt-ids", "--prompt-ids", dest="prompt_ids", default="",
+                    help="token ids (blanks or commas between them), also where the folder has a tokenizer")
+    ap.add_argument("-prompt-file", "--prompt-file", dest="prompt_file", default="",
+                    help="a file with one prompt a line (in the place of -prompt)")
+    ap.add_argument("-n", "--n", "-len", "--len", "-max-new-tokens", "--max-new-tokens", dest="n", type=int,
+                    default=20, help="number of tokens to generate")
+    ap.add_argument("-stop-id", "--stop-id", dest="stop_ids", type=int, action="append", default=[],
+                    help="a token id that ends a sequence, beside the configuration's (may be given several times)")
     ap.add_argument("-kv-cache-size", "--kv-cache-size", dest="kv_cache_size", type=int, default=2048,
                     help="tokens the cache holds for each sequence of the batch")
     ap.add_argument("-temp", "--temp", type=float, default=0.7, help="temperature (0 = greedy)")
@@ -61,7 +70,19 @@ def main(argv: Optional[List[str]] = None) -> int:
 
     import longbow_quarrel_amd as lq
 
-    prompts_text = args.prompt.split("|")
+    as_ids = bool(args.prompt_ids)
+    if args.prompt_file:
+        try:
+            with open(args.prompt_file) as f:
+                prompts_text = [line.strip() for line in f if line.strip()]
+        except OSError as e:
+            print(f"Error: cannot read --prompt-file: {e}", file=sys.stderr)
+            return 1
+        if not prompts_text:
+            print(f"Error: {args.prompt_file} holds no prompt", file=sys.stderr)
+            return 1
+    else:
+        prompts_text = (args.prompt_ids or args.prompt).split("|")
     max_tokens = args.kv_cache_size * max(1, len(prompts_text))
     t0 = time.perf_counter()
     tokenizer = None
@@ -87,7 +108,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     if args.verbose:
         print(f"loaded in {time.perf_counter() - t0:.2f}s")
 
-    prompts = [_encode(p.strip(), tokenizer, spec.bos_id) for p in prompts_text]
+    prompts = [_encode(p.strip(), None if as_ids else tokenizer, spec.bos_id) for p in prompts_text]
     params = lq.SamplingParams(temperature=args.temp, top_k=args.topk, top_p=args.topp,
                                repetition_penalty=args.penalty, seed=args.seed)
 
@@ -103,7 +124,7 @@ def main(argv: Optional[List[str]] = None) -> int:
             print(prefix + show([token]), end=" ", flush=True)
 
     start = time.perf_counter()
-    result = lq.generate(engine, prompts, args.n, params, callback=callback)
+    result = lq.generate(engine, prompts, args.n, params, callback=callback, extra_stop_ids=args.stop_ids)
     duration = time.perf_counter() - start
     if args.stream:
         print(" [END]")

@@ -9,6 +9,7 @@ int lq_attention_generic(const void* q, int ldq, void* out, int ldo, int dtype, 
 bool lq_attention_mfma_accepts(int dtype, int nh, int nkv, int hd, int block_size, int ldq, int ldo,
                                const void* q, const void* out, int decode);
 long long lq_attention_mfma_workspace(int rows, int nh, int nkv, int hd, int max_len);
+int lq_attention_mfma_unit_search(const int* pos, int rows, int nkv, int max_len);
 int lq_attention_mfma(const void* q, int ldq, void* out, int ldo, int rows, int batch, int nh, int nkv,
                       int hd, const int* row_pos, const int* seq_slot, const int* cu_rows,
                       const int* block_table, int bt_stride, const void* kcache, const void* vcache,
@@ -23,6 +24,32 @@ extern "C" long long lq_attention_workspace(int dtype, int rows, int nh, int nkv
   if (!decode || dtype != LQ_BF16) return 0;
   if (!lq_attention_mfma_accepts(dtype, nh, nkv, hd, block_size, 8, 8, nullptr, nullptr, decode)) return 0;
   return lq_attention_mfma_workspace(rows, nh, nkv, hd, max_len);
+}
+
+// A decoding launch shapes its grid by the bound of the lengths rounded up to this many tokens: whoever keeps
+// launches for replay (a captured step) needs a new one only when the longest sequence passes a multiple of it.
+extern "C" int lq_attention_length_bucket() { return LQ_DECODE_LENGTH_BUCKET; }
+
+// Whether the sequences of a decoding launch differ so much in length (the longest at least half again as long as
+// their mean, and 512 tokens or more: below that there is nothing to share out) that the launch does better
+// sharing the keys out by the true lengths (`uneven` of lq_attention) than cutting every sequence as if it were
+// the longest.  With equal lengths that scheme costs 1 to 3 %, which is why it waits for this answer.
+extern "C" int lq_attention_lengths_uneven(const int* lengths, int n) {
+  if (lengths == nullptr || n < 2) return 0;
+  long long longest = 0, sum = 0;
+  for (int i = 0; i < n; ++i) {
+    sum += lengths[i];
+    if (lengths[i] > longest) longest = lengths[i];
+  }
+  return longest >= 512 && 2 * (long long)n * longest >= 3 * sum;
+}
+
+// For tests, on the host: how many tries the units of an `uneven` decoding launch need to find their split
+// length for sequences whose newest positions are pos[0..rows) (0: such a launch does not take that way; -1:
+// they would not find it, which must not happen for positions below max_len).
+extern "C" int lq_attention_unit_search(const int* pos, int rows, int nkv, int max_len) {
+  if (pos == nullptr || rows <= 0 || nkv <= 0 || max_len <= 0) return 0;
+  return lq_attention_mfma_unit_search(pos, rows, nkv, max_len);
 }
 
 // Whether a decoding launch can take the rotation of q and k and the cache write upon itself

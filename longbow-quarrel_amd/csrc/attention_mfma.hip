@@ -785,7 +785,17 @@ __device__ inline int wave_prefix_sums(int v) {
   return v;
 }
 
-__device__ inline bool balanced_item(const AttnArgs& a, int u, DecodeItem& it) {
+// Splits of length 256 k that hold keys of a sequence whose newest position is `pos` (position p lies in block
+// p / 256; blocks of 256 positions and their quotients are small integers, which a float division gives exactly).
+// One function for the kernel's search and for the host's check of it.
+__host__ __device__ inline int splits_with_keys(int pos, int k) {
+  return (int)(((float)(pos >> 8) + 0.5f) / (float)k) + 1;
+}
+constexpr int UNIT_SEARCH_TRIES = 1024;
+
+// -> 1: unit u has work (in `it`); 0: it has none; -1: no split length was found within the tries, which the
+// host's choice of the units rules out (decode_units) as long as the lengths lie within the launch's bound.
+__device__ inline int balanced_item(const AttnArgs& a, int u, DecodeItem& it) {
   const int lane = threadIdx.x & 63;
   const bool mine = lane < a.batch;
   const int pl = mine ? a.row_pos[lane] : -1;  // lane l looks after sequence l (at most 64 of them)
@@ -793,10 +803,9 @@ __device__ inline bool balanced_item(const AttnArgs& a, int u, DecodeItem& it) {
   const int total = __builtin_amdgcn_readlane(wave_prefix_sums(pl + 1), 63);
   // the smallest multiple of 256 with which the splits that hold keys are no more than the units; blocks of
   // 256 positions and their quotients are small integers, which a float division gives exactly
-  const float blocks = (float)(pl >> 8) + 0.5f;  // (position p lies in block p / 256)
   int k = max(1, (total + 256 * a.units - 1) / (256 * a.units)), cnt = 0;
-  for (int tries = 0; tries < 1024; ++tries, ++k) {
-    cnt = mine ? (int)(blocks / (float)k) + 1 : 0;  // splits of this lane's sequence that hold keys
+  for (int tries = 0; tries < UNIT_SEARCH_TRIES; ++tries, ++k) {
+    cnt = mine ? splits_with_keys(pl, k) : 0;  // splits of this lane's sequence that hold keys
     if (__builtin_amdgcn_readlane(wave_prefix_sums(cnt), 63) <= a.units) break;
   }
   const int SL = 256 * k;
@@ -805,7 +814,8 @@ __device__ inline bool balanced_item(const AttnArgs& a, int u, DecodeItem& it) {
   const int part = mine && (pl + 1) % SL != 0 ? 1 : 0, full = cnt - part;
   const int full_incl = wave_prefix_sums(full), part_incl = wave_prefix_sums(part);
   const int n_full = __builtin_amdgcn_readlane(full_incl, 63), n_part = __builtin_amdgcn_readlane(part_incl, 63);
-  if (n_full + n_part > a.units || u >= n_full + n_part) return false;  // (the first cannot be: see decode_units)
+  if (n_full + n_part > a.units) return -1;
+  if (u >= n_full + n_part) return 0;
   const bool whole = u < n_full;
   const int row = whole ? __popcll(__ballot(mine && full_incl <= u))
                         : __popcll(__ballot(mine && part_incl <= u - n_full));
@@ -817,7 +827,7 @@ __device__ inline bool balanced_item(const AttnArgs& a, int u, DecodeItem& it) {
   it.first_unit = __builtin_amdgcn_readlane(full_incl - full, row);
   it.last_unit = n_full + __builtin_amdgcn_readlane(part_incl - part, row);
   it.split = whole ? u - it.first_unit : it.n_full;
-  return true;
+  return 1;
 }
 
 template <int HD, int NW, bool PIECES = false>
@@ -834,7 +844,19 @@ __global__ __launch_bounds__(NW * 64, (HD <= 128 ? 2 : 1)) void attn_heads_kerne
   if (a.units > 0) {
     DecodeItem it;
     kvh = blockIdx.x;
-    if (!balanced_item(a, blockIdx.y, it)) return;  // the whole block: more units than splits with keys
+    const int found = balanced_item(a, blockIdx.y, it);
+    if (found < 0) {
+      // Nobody would write the output: make that loud instead of leaving what the buffer held.  Units 0 ..
+      // batch - 1 (there are at least two a sequence) fill their row's heads of this kv head with NaN.
+      if ((int)blockIdx.y < a.batch) {
+        bf16_t nan;
+        nan.bits = 0x7FC0;
+        bf16_t* o = a.out + (long long)blockIdx.y * a.ldo + (long long)kvh * G * HD;
+        for (int i = threadIdx.x; i < G * HD; i += NW * 64) o[i] = nan;
+      }
+      return;
+    }
+    if (found == 0) return;  // the whole block: more units than splits with keys
     b = it.row;
     p = it.pos;
     slot = it.slot;
@@ -1169,10 +1191,10 @@ bool lq_attention_mfma_accepts(int dtype, int nh, int nkv, int hd, int block_siz
 // for the waiting (33 to 63 long sequences, which one workgroup each would put two on some units and one on
 // others), and of two lengths that come to the same the shorter (more waves to hide each other's round
 // trips).  It depends on the
-// bound rounded up to 1024, so that launches whose bounds differ less than that add up their sums in the same
+// bound rounded up to LQ_DECODE_LENGTH_BUCKET, so that launches whose bounds differ less than that add up their sums in the same
 // order.
 static int decode_split_len(int rows, int nkv, int max_len) {
-  const long long bound = (long long)lq_ceil_div(max_len, 1024) * 1024;
+  const long long bound = (long long)lq_ceil_div(max_len, LQ_DECODE_LENGTH_BUCKET) * LQ_DECODE_LENGTH_BUCKET;
   // (asked for at every launch: the answers are kept)
   static std::mutex guard;
   static std::map<std::tuple<int, int, long long>, int> known;
@@ -1215,7 +1237,7 @@ static int decode_split_len(int rows, int nkv, int max_len) {
 #endif
 static int decode_units(int rows, int nkv, int max_len, int window) {
   if (window > 0 || rows < 2 || rows > 64) return 0;
-  const long long bound = (long long)lq_ceil_div(max_len, 1024) * 1024;
+  const long long bound = (long long)lq_ceil_div(max_len, LQ_DECODE_LENGTH_BUCKET) * LQ_DECODE_LENGTH_BUCKET;
   long long by_cap = MAX_DECODE_BLOCKS / nkv;
   if (by_cap < 2 * rows) by_cap = (long long)LQ_UNITS_A_SEQUENCE * rows;
   const long long by_bound = (long long)rows * (bound / 256);
@@ -1225,6 +1247,25 @@ static int decode_units(int rows, int nkv, int max_len, int window) {
   // that; it gives the search 1 024 steps.
   if (rows * bound / (256 * units) > 512) return 0;
   return (int)units;
+}
+
+// The host's check of the search that the kernel's units make for their split length (balanced_item): the tries
+// it takes for sequences whose newest positions are `pos[0..rows)`, or -1 if it does not end within
+// UNIT_SEARCH_TRIES (which the choice of the units is meant to rule out), or 0 where the launch would not take
+// the units' way at all.  The same arithmetic, one sequence after another instead of a lane each.
+int lq_attention_mfma_unit_search(const int* pos, int rows, int nkv, int max_len) {
+  const int units = decode_units(rows, nkv, max_len, 0);
+  if (units <= 0) return 0;
+  long long total = 0;
+  for (int i = 0; i < rows; ++i) total += pos[i] + 1;
+  int k = (int)((total + 256LL * units - 1) / (256LL * units));
+  if (k < 1) k = 1;
+  for (int tries = 0; tries < UNIT_SEARCH_TRIES; ++tries, ++k) {
+    long long cnt = 0;
+    for (int i = 0; i < rows; ++i) cnt += splits_with_keys(pos[i], k);
+    if (cnt <= units) return tries + 1;
+  }
+  return -1;
 }
 
 // Floats of workspace a decode launch needs (0 when one split is enough): enough for either grid, the

@@ -124,5 +124,8 @@ int lq_compute_units();  // of the current device
     }                                                                    \
   } while (0)
 
+// tokens by which a decoding attention launch rounds the bound of the lengths up before it shapes its grid
+#define LQ_DECODE_LENGTH_BUCKET 1024
+
 static inline int lq_ceil_div(int a, int b) { return (a + b - 1) / b; }
 static inline long long lq_ceil_div64(long long a, long long b) { return (a + b - 1) / b; }

@@ -20,4 +20,7 @@
 // Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
 // threads) race; calls on one stream, or ordered by events, do not.  Nothing in the array has to start
 // at zero (the first stage writes every entry that the second reads), so it is never cleared.
+// The first call on a device asks the runtime for that device's address of the array (under a lock,
+// once): make that call before a stream capture begins, since the query is no stream work and a
+// capture may refuse it; every later call on the device only launches the two kernels.
 extern "C" int lq_argmax_no_alloc(const float* logits, int ld, int rows, int V, int* out, hipStream_t stream);

@@ -1151,6 +1151,10 @@ __global__ void advance_kernel(int* row_pos, int* seq_start, int* seq_len, int b
 
 }  // namespace
 
+// Ids of a sequence's history that the repetition penalty looks at: the width of the ring that lq_apply_penalty,
+// lq_argmax and lq_sample take (whoever allocates the ring asks here).
+extern "C" int lq_penalty_window() { return RECENT; }
+
 extern "C" int lq_apply_penalty(float* logits, int ld, int rows, int V, const int* seq_slot, const int* recent,
                                 const int* recent_n, float penalty, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && V > 0 && ld >= V, "penalty: bad sizes");

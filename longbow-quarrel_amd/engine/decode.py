@@ -10,9 +10,11 @@ the block tables ahead of the lengths and reads the sampled tokens back.
 
 A graph bakes in the pointers of the workspace, the logits buffer and its own integer
 arrays; the cache, the weights and the sampler state have fixed addresses for the
-life of the engine.  The split grid of the attention kernel depends on an upper
-bound of the lengths, so a graph is keyed by (B, bound) and a new one is captured
-when a sequence outgrows the bound.
+life of the engine.  What a mixer's launches depend on beside the batch size (for
+attention: an upper bound of the lengths, which shapes its split grid, and whether the
+lengths differ much) the mixers say themselves (`Engine.length_bound`,
+`Engine.lengths_uneven`); a graph is keyed by (B, bound, uneven) and a new one is
+captured when a sequence outgrows the bound.
 
 The graphs of one `DecodeGraphs` replay one at a time on one stream, so they share one
 workspace and one logits buffer, as large as the largest of them needs; when a new
@@ -29,8 +31,6 @@ from ..kernels.dry import DryKernels
 from ..parts.base import StepContext, Workspace
 from ..sampling.sampler import Sampler
 
-LEN_BUCKET = 1024
-
 
 def _pad4(n: int) -> int:
     return (n + 3) // 4 * 4
@@ -42,7 +42,7 @@ class DecodeGraph:
         self.engine = engine
         self.batch = batch
         self.bound = bound
-        self.uneven = uneven  # the step's hint to the attention kernel (`lengths_uneven`), fixed at capture
+        self.uneven = uneven  # the step's hint to the attention kernel (`Engine.lengths_uneven`), fixed at capture
         dev = engine.device
         b = batch
         self.sizes = [b, b, b, b, b, b, b + 1, b]  # tokens row_seq row_pos slot start len cu want

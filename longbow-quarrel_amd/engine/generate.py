@@ -16,9 +16,11 @@ or the caller and every sampled token is checked.
 `GenerationLoop` holds the decisions only and talks to a backend with a handful of
 methods, so that the decisions can be tested without a GPU; `EngineBackend` is the
 real one.  It feeds a batch's prompts in portions of at most `max_prefill_rows` rows
-(the step's workspace grows with its rows, not with the batch), and it reports a row of
-logits that holds a NaN or an infinity as `NonFiniteLogits` where the reference takes
-the first finite index (internal/engine/sampler.go:72-75, 107-123).  Replayed decoding steps
+(the step's workspace grows with its rows, not with the batch).  A row of logits that holds a
+NaN or an infinity is not sampled from, where the reference takes the first finite index
+(internal/engine/sampler.go:72-75, 107-123): that request ends there (finish "error"), the
+others of its batch and the batches after it run to their ends, and then the call raises
+`NonFiniteLogits`, which names the requests and carries everybody's tokens as `result`.  Replayed decoding steps
 are queued one ahead of the host (`_Launched`, `EngineBackend.ahead`): the device goes from one
 step to the next without waiting for the loop's decisions, which arrive a step late and are
 applied to the step that is already there.
@@ -34,15 +36,15 @@ import torch
 from ..cache import BLOCK_SIZE, CacheFull
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import NonFiniteLogits, Sampler
-from ..sampling.state import SamplerState, sequence_key
-from .decode import LEN_BUCKET, DecodeGraphs
-from .step import Engine, SequenceTooLong, StepEntry, lengths_uneven
+from ..sampling.state import RECENT, SamplerState, sequence_key
+from .decode import DecodeGraphs
+from .step import Engine, SequenceTooLong, StepEntry
 
 
 @dataclass
 class GenerationResult:
     tokens: List[List[int]]  # generated ids per request, in the order of the prompts (prompts not included)
-    finish: List[str]  # "stop" | "length" for each request
+    finish: List[str]  # "stop" | "length" for each request ("error": its logits held a NaN or an infinity)
     prefill_seconds: float = 0.0
     decode_seconds: float = 0.0
     prefill_tokens: int = 0
@@ -138,6 +140,7 @@ class GenerationLoop:
         limit = self._token_limits(prompts, max_new_tokens)
         pending = list(range(n))
         be = self.backend
+        faulty: List[str] = []
         while pending:
             batch = self._next_batch(pending, prompts, limit)
             pending = pending[len(batch):]
@@ -157,6 +160,11 @@ class GenerationLoop:
                     survivors: List[int] = []
                     for r, tok in zip(live, sampled):
                         tok = int(tok)
+                        if tok < 0:  # no token: the row's logits were not finite
+                            result.finish[r] = "error"
+                            faulty.append(f"request {r} (slot {slots[r]})")
+                            be.release(slots.pop(r))
+                            continue
                         if tok in stops:
                             result.finish[r] = "stop"
                             if include_stop:
@@ -189,6 +197,9 @@ class GenerationLoop:
             finally:
                 for s in slots.values():
                     be.release(s)
+        if faulty:
+            raise NonFiniteLogits(f"the logits of {', '.join(faulty)} hold a NaN or an infinity; nothing was sampled "
+                                  "from them (the other requests ran on: see .result)", result)
         return result
 
 
@@ -204,13 +215,13 @@ class EngineBackend:
         self.params = params
         self.max_prefill_rows = int(max_prefill_rows)
         if not hasattr(engine, "sampler_state"):
-            engine.sampler_state = SamplerState(engine.cache.max_slots, engine.device)
+            engine.sampler_state = SamplerState(engine.cache.max_slots, engine.device,
+                                                window=getattr(engine.kernels, "penalty_window", RECENT))
         self.sampler = Sampler(engine.kernels, engine.sampler_state, params)
         self.use_graphs = use_graphs and engine.graph_safe and \
             (engine.device.type == "cuda" or graphs_cls is not DecodeGraphs)
         self.graphs = graphs_cls(engine, self.sampler) if self.use_graphs else None
         self.current = None  # the graph whose arrays hold the live batch, as the last step left them
-        self.request_of: Dict[int, int] = {}  # slot -> index of the request that runs there
         # a copy of each step's logits: before sampling where steps run directly, as the sampler left them
         # (with the repetition penalty applied, if there is one) where they are replayed from a graph
         self.keep_logits = False
@@ -247,12 +258,10 @@ class EngineBackend:
         self._drop_ahead()
         slot = self.engine.new_sequence()
         self.engine.sampler_state.start(slot, sequence_key(self.params.seed, request_index), prompt)
-        self.request_of[slot] = request_index
         self.current = None  # whatever a graph's arrays hold is of an earlier batch
         return slot
 
     def release(self, slot: int) -> None:
-        self.request_of.pop(slot, None)
         self.engine.release(slot)
 
     def prefill(self, slots: Sequence[int], prompts: Sequence[Sequence[int]]) -> List[int]:
@@ -296,17 +305,9 @@ class EngineBackend:
         # waits for its tokens before it does anything else with the sequences: no waits between streams.
         # (What is queued ahead is waited for in `_drop_ahead` before other work may touch its slots.)
         step = e.run_on_stream(lambda: self._decode_graph(list(slots), list(last_tokens), changed), handshake=False)
-        return self._checked(step.tokens(list(slots)), slots)
+        return step.tokens(list(slots))  # (-1 where a row's logits were not finite: the loop ends that request)
 
     # ---- internals ------------------------------------------------------------------------
-    def _checked(self, tokens: List[int], slots: Sequence[int]) -> List[int]:
-        """The sampler's answer for a row of logits with a NaN or an infinity is no token."""
-        bad = [s for s, t in zip(slots, tokens) if t < 0]
-        if bad:
-            names = ", ".join(f"request {self.request_of.get(s, '?')} (slot {s})" for s in bad)
-            raise NonFiniteLogits(f"the logits of {names} hold a NaN or an infinity; nothing was sampled from them")
-        return tokens
-
     def _sample_eager(self, logits: torch.Tensor, slots: Sequence[int]) -> List[int]:
         e = self.engine
 
@@ -318,7 +319,7 @@ class EngineBackend:
             self.sampler.sample(logits, seq_slot, out)
             return out.cpu().tolist()
 
-        return self._checked(e.run_on_stream(body), slots)
+        return e.run_on_stream(body)
 
     def _decode_graph(self, slots: List[int], last_tokens: List[int], changed: bool) -> "_Launched":
         """The launched step whose tokens answer this call: the one queued ahead if it is the step asked
@@ -345,9 +346,9 @@ class EngineBackend:
         cache = e.cache
         starts = [cache.length(s) for s in slots]
         longest = max(starts) + 1
-        bound = (longest + LEN_BUCKET - 1) // LEN_BUCKET * LEN_BUCKET
+        bound = e.length_bound(longest)
         growth = {s: 1 for s in slots}
-        uneven = lengths_uneven([n + 1 for n in starts])
+        uneven = e.lengths_uneven([n + 1 for n in starts])
         if same_graph is not None:
             if bound != same_graph.bound or uneven != same_graph.uneven:
                 return None

@@ -21,20 +21,12 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..cache import CacheManager
 from ..model import DecoderModel
 from ..parts.base import BuildEnv, StepContext, Workspace
-
-
-def lengths_uneven(lengths: Sequence[int]) -> bool:
-    """Whether the sequences of a decoding step differ so much in length (the longest at least half again
-    as long as their mean) that the attention kernel does better sharing the keys out by the true lengths
-    than cutting every sequence as if it were the longest; below 512 tokens there is nothing to share out.
-    The one place where this is decided, from the lengths alone, for direct and for captured steps alike,
-    so that both sum in the same order."""
-    return len(lengths) >= 2 and max(lengths) >= 512 and 2 * len(lengths) * max(lengths) >= 3 * sum(lengths)
 
 
 class SequenceTooLong(ValueError):
@@ -53,12 +45,16 @@ def _pad4(n: int) -> int:
 
 
 class StepMeta:
-    """Packs a step's integer arrays into one host buffer and one upload."""
+    """Packs a step's integer arrays into one pinned host buffer and one upload.  Two host buffers take
+    turns, each with an event behind its copy, so that the upload does not wait for the device and a
+    buffer is not written again before its last copy has been taken."""
 
     def __init__(self, device: torch.device) -> None:
         self.device = device
         self.cap = 0
-        self.host: Optional[torch.Tensor] = None
+        self.hosts: List[torch.Tensor] = []
+        self.events: List[Optional["torch.cuda.Event"]] = [None, None]
+        self.turn = 0
         self.dev: Optional[torch.Tensor] = None
 
     def _grow(self, n: int) -> None:
@@ -66,21 +62,37 @@ class StepMeta:
             return
         self.cap = max(1024, int(n * 1.5))
         pin = self.device.type == "cuda"
-        self.host = torch.empty(self.cap, dtype=torch.int32, pin_memory=pin)
+        for ev in self.events:
+            if ev is not None:
+                ev.synchronize()
+        self.events = [None, None]
+        self.hosts = [torch.empty(self.cap, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
         self.dev = torch.empty(self.cap, dtype=torch.int32, device=self.device)
 
-    def upload(self, sections: Sequence[Sequence[int]]) -> List[torch.Tensor]:
-        sizes = [len(s) for s in sections]
-        total = sum(_pad4(max(1, n)) for n in sizes)
+    def upload(self, sections: Sequence[np.ndarray]) -> List[torch.Tensor]:
+        """`sections`: integer arrays; each gets a run of the device buffer (16-byte aligned, at least
+        one entry long).  -> the device views, in order."""
+        sizes = [int(s.size) for s in sections]
+        offsets, total = [], 0
+        for n in sizes:
+            offsets.append(total)
+            total += _pad4(max(1, n))
         self._grow(total)
-        flat: List[int] = []
-        offsets = []
-        for s, n in zip(sections, sizes):
-            offsets.append(len(flat))
-            flat.extend(s)
-            flat.extend([0] * (_pad4(max(1, n)) - n))
-        self.host[:total] = torch.tensor(flat, dtype=torch.int32)
-        self.dev[:total].copy_(self.host[:total])
+        self.turn ^= 1
+        if self.events[self.turn] is not None:
+            self.events[self.turn].synchronize()
+        host = self.hosts[self.turn]
+        flat = host.numpy()
+        for s, o, n in zip(sections, offsets, sizes):
+            flat[o : o + n] = s
+            flat[o + n : o + _pad4(max(1, n))] = 0
+        if self.device.type == "cuda":
+            self.dev[:total].copy_(host[:total], non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            self.events[self.turn] = ev
+        else:
+            self.dev[:total].copy_(host[:total])
         return [self.dev[o : o + max(1, n)] for o, n in zip(offsets, sizes)]
 
 
@@ -95,6 +107,9 @@ class Engine:
         self.env = env
         self.kernels = env.kernels
         self.device = env.device
+        prepare = getattr(env.kernels, "prepare", None)
+        if prepare is not None:
+            prepare(env.device)
         self.dtype = env.dtype
         self.vocab_size = model.spec.vocab_size
         self.cache = CacheManager(model.cache_needs(), max_tokens, max_slots, env.dtype, env.device)
@@ -122,25 +137,46 @@ class Engine:
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
 
+    # ---- what a decoding step's launches depend on beside its batch size ----------------------
+    def length_bound(self, longest: int) -> int:
+        """The bound of the lengths that a decoding step is shaped for when its longest sequence holds
+        `longest` tokens (the mixers' answer: `Mixer.length_bound`)."""
+        return self.model.length_bound(self.kernels, longest)
+
+    def lengths_uneven(self, lengths: Sequence[int]) -> bool:
+        """Whether a decoding step with these lengths is to be marked `uneven` (the mixers' answer:
+        `Mixer.lengths_uneven`); asked here for direct and for captured steps alike, so that both sum
+        in the same order."""
+        return self.model.lengths_uneven(self.kernels, lengths)
+
     # ---- the step --------------------------------------------------------------------------
-    def _validate(self, entries: Sequence[StepEntry]) -> None:
+    def _validate(self, entries: Sequence[StepEntry]) -> List[np.ndarray]:
+        """Refuses a step that cannot run, before anything changes.  -> each entry's tokens as an array."""
         if not entries:
             raise ValueError("a step needs at least one sequence")
         seen = set()
+        arrays: List[np.ndarray] = []
         for e in entries:
             if e.slot in seen:
                 raise ValueError(f"slot {e.slot} appears twice in one step")
             seen.add(e.slot)
             held = self.cache.length(e.slot)  # raises if the slot is not in use
-            if len(e.tokens) == 0:
+            try:
+                t = np.asarray(e.tokens, dtype=np.int64).reshape(-1)
+            except (TypeError, ValueError, OverflowError):
+                raise ValueError(f"slot {e.slot}: token ids must be integers") from None
+            if t.size == 0:
                 raise ValueError(f"slot {e.slot}: a step entry needs at least one token")
-            self.check_room(e.slot, held, len(e.tokens))
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise ValueError(f"slot {e.slot}: token id {t} is outside the vocabulary [0, {self.vocab_size})")
+            self.check_room(e.slot, held, int(t.size))
+            low, high = int(t.min()), int(t.max())
+            if low < 0 or high >= self.vocab_size:
+                bad = low if low < 0 else high
+                raise ValueError(f"slot {e.slot}: token id {bad} is outside the vocabulary [0, {self.vocab_size})")
             for w in e.want:
-                if not 0 <= int(w) < len(e.tokens):
-                    raise ValueError(f"slot {e.slot}: wanted place {w} is outside its {len(e.tokens)} tokens")
+                if not 0 <= int(w) < t.size:
+                    raise ValueError(f"slot {e.slot}: wanted place {w} is outside its {t.size} tokens")
+            arrays.append(t)
+        return arrays
 
     def check_room(self, slot: int, held: int, new: int) -> None:
         limit = self.max_sequence_tokens
@@ -172,8 +208,8 @@ class Engine:
         """Runs the entries' tokens; returns float32 logits [wanted, vocab] in the order of the
         entries and of each entry's `want` (None if nothing is wanted).  `observe(name, x, pending)`, for
         debugging, sees the residual stream after the embedding and after every run of the schedule."""
-        self._validate(entries)
-        return self.run_on_stream(lambda: self._step(entries, observe))
+        arrays = self._validate(entries)
+        return self.run_on_stream(lambda: self._step(entries, arrays, observe))
 
     def make_context(self, ws: Workspace, arrays: Sequence[torch.Tensor], slots: Sequence[int],
                      starts: Sequence[int], new: Sequence[int], max_len: int, logits_out=None, observe=None,
@@ -182,7 +218,7 @@ class Engine:
         `arrays`: the device arrays tokens, row_seq, row_pos, seq_slot, seq_start, seq_len, cu_rows;
         `slots`, `starts`, `new`: per sequence, on the host (`starts` may be empty where the lengths
         live on the device only, as in a captured step); `max_len`: an upper bound of the lengths after
-        the step; `uneven`: whether a decoding step's sequences differ much in length (`lengths_uneven`)."""
+        the step; `uneven`: whether a decoding step's sequences differ much in length (`Engine.lengths_uneven`)."""
         tokens, row_seq, row_pos, seq_slot, seq_start, seq_len, cu_rows = arrays
         return StepContext(
             kernels=kernels if kernels is not None else self.kernels, dtype=self.dtype, device=self.device, ws=ws,
@@ -195,36 +231,33 @@ class Engine:
         """The model over one step's rows, from this engine's cache."""
         return self.model.forward(ctx, self.cache.layer_views(), want_rows, n_want)
 
-    def _step(self, entries: Sequence[StepEntry], observe=None) -> Optional[torch.Tensor]:
+    def _step(self, entries: Sequence[StepEntry], arrays: Sequence[np.ndarray], observe=None) -> Optional[torch.Tensor]:
         cache = self.cache
-        growth = {e.slot: len(e.tokens) for e in entries}
+        new = [int(a.size) for a in arrays]
+        growth = {e.slot: n for e, n in zip(entries, new)}
         cache.reserve(growth)  # CacheFull leaves everything as it was
 
-        tokens: List[int] = []
-        row_seq: List[int] = []
-        row_pos: List[int] = []
-        want_rows: List[int] = []
-        slots, starts, lens, cu = [], [], [], [0]
-        for b, e in enumerate(entries):
-            n0 = cache.length(e.slot)
-            n = len(e.tokens)
-            base = len(tokens)
-            tokens.extend(int(t) for t in e.tokens)
-            row_seq.extend([b] * n)
-            row_pos.extend(range(n0, n0 + n))
-            want_rows.extend(base + int(w) for w in e.want)
-            slots.append(e.slot)
-            starts.append(n0)
-            lens.append(n0 + n)
-            cu.append(len(tokens))
+        # the step's arrays, whole vectors at a time: no work per token on the host
+        batch = len(entries)
+        slots = [e.slot for e in entries]
+        starts = [cache.length(s) for s in slots]
+        counts = np.asarray(new, dtype=np.int64)
+        cu = np.zeros(batch + 1, dtype=np.int64)
+        np.cumsum(counts, out=cu[1:])
+        rows = int(cu[-1])
+        first = np.asarray(starts, dtype=np.int64)
+        row_seq = np.repeat(np.arange(batch, dtype=np.int64), counts)
+        row_pos = np.arange(rows, dtype=np.int64) + np.repeat(first - cu[:-1], counts)
+        tokens = arrays[0] if batch == 1 else np.concatenate(arrays)
+        want_rows = np.asarray([int(cu[b]) + int(w) for b, e in enumerate(entries) for w in e.want], dtype=np.int64)
+        lens = [a + n for a, n in zip(starts, new)]
         d_tokens, d_row_seq, d_row_pos, d_slot, d_start, d_len, d_cu, d_want = self.meta.upload(
-            [tokens, row_seq, row_pos, slots, starts, lens, cu, want_rows])
+            [tokens, row_seq, row_pos, np.asarray(slots), first, np.asarray(lens), cu, want_rows])
 
         self.ws.reset()
         ctx = self.make_context(self.ws, (d_tokens, d_row_seq, d_row_pos, d_slot, d_start, d_len, d_cu), slots,
-                                starts, [len(e.tokens) for e in entries], max(lens), observe=observe,
-                                uneven=lengths_uneven(lens))
-        logits = self.forward(ctx, d_want, len(want_rows))
+                                starts, new, max(lens), observe=observe, uneven=self.lengths_uneven(lens))
+        logits = self.forward(ctx, d_want, int(want_rows.size))
         cache.advance(growth)
         self.steps_run += 1
         return logits

@@ -80,7 +80,22 @@ class HipKernels:
         self.force_generic = False  # route linear and attention to the size-agnostic kernels
         # ticket counters of the decoding attention (one for each row and kv head of a launch); a launch
         # finds them zero and leaves them zero, so launches through one object must not overlap
-        self._tickets = torch.zeros(1 << 18, dtype=torch.int32, device="cuda")
+        self._tickets: dict = {}  # device -> the counters
+
+    def prepare(self, device: torch.device) -> None:
+        """What an engine asks once before its first step on `device`: everything that this object allocates
+        by itself is there afterwards, so that no launch under a stream capture has to allocate."""
+        self.tickets(device)
+
+    def tickets(self, device: torch.device) -> torch.Tensor:
+        """The ticket counters on `device` (made at the first launch there, or by `prepare`)."""
+        device = torch.device(device)
+        if device.index is None:
+            device = torch.device(device.type, torch.cuda.current_device())
+        t = self._tickets.get(device)
+        if t is None:
+            t = self._tickets[device] = torch.zeros(1 << 18, dtype=torch.int32, device=device)
+        return t
 
     # ------------------------------------------------------------------ plumbing
     def use_stream(self, stream: Optional["torch.cuda.Stream"]) -> None:
@@ -427,6 +442,21 @@ class HipKernels:
         shares K over blocks (`linear_pieces` > 1), and adds them up itself."""
         return self.attention_folds_rope(dtype, heads, kv_heads, head_dim, block_size)
 
+    @query
+    def decode_length_bound(self, longest: int) -> int:
+        """The bound of the lengths that a decoding `attention` launch shapes its grid by when the longest
+        sequence holds `longest` tokens: launches with one bound sum in one order, so a step kept for replay
+        serves until a sequence outgrows its bound."""
+        bucket = int(self.lib.lq_attention_length_bucket())
+        return (max(1, int(longest)) + bucket - 1) // bucket * bucket
+
+    @query
+    def decode_lengths_uneven(self, lengths) -> bool:
+        """Whether a decoding step with these lengths should tell `attention` that they differ much
+        (`uneven`): the kernel library's own rule."""
+        n = len(lengths)
+        return bool(self.lib.lq_attention_lengths_uneven((c_int * max(1, n))(*[int(x) for x in lengths]), c_int(n)))
+
     def rope_table(self, freqs: torch.Tensor, row_pos: torch.Tensor, out: torch.Tensor) -> None:
         """out[r, i] = (cos, sin) of row_pos[r] * freqs[i]; float32 [rows, pairs, 2]."""
         self._dev(freqs, row_pos, out)
@@ -493,13 +523,14 @@ class HipKernels:
             if cos_sin.dtype != torch.float32 or tuple(cos_sin.shape) != (rows, head_dim // 2, 2) or not cos_sin.is_contiguous():
                 raise KernelLibraryError("attention: cos_sin must be dense float32 [rows, head_dim/2, 2]")
             ldk, ldv = self._rows2d(k_new, "k_new"), self._rows2d(v_new, "v_new")
+        tickets = self.tickets(q.device)
         rc = self.lib.lq_attention(
             _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")),
             c_int(_code(out)), c_int(rows), c_int(batch), c_int(heads), c_int(kv_heads), c_int(head_dim),
             _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(cu_rows), _ptr(block_table),
             c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
             c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
-            c_longlong(ws_n), _ptr(self._tickets), c_longlong(self._tickets.numel()), _ptr(k_new if cos_sin is not None else None),
+            c_longlong(ws_n), _ptr(tickets), c_longlong(tickets.numel()), _ptr(k_new if cos_sin is not None else None),
             _ptr(v_new if cos_sin is not None else None), c_int(ldk), c_int(ldv), _ptr(cos_sin),
             c_int(1 if uneven and decode else 0), c_int(pieces), c_longlong(piece_stride),
             c_int(1 if self.force_generic else 0), self.stream)
@@ -509,11 +540,16 @@ class HipKernels:
             # the error goes up
             message = self.lib.lq_last_error().decode("utf-8", "replace")
             try:
-                self._tickets.zero_()
+                tickets.zero_()
             finally:
                 raise KernelLibraryError(message)
 
     # ------------------------------------------------------------------ sampling
+    @property
+    def penalty_window(self) -> int:
+        """Width of the ring of recent ids that the sampling kernels take (the library's constant)."""
+        return int(self.lib.lq_penalty_window())
+
     def apply_penalty(self, logits: torch.Tensor, seq_slot: torch.Tensor, recent: torch.Tensor,
                       recent_n: torch.Tensor, penalty: float) -> None:
         """Repetition penalty on the distinct ids in each sequence's ring of recent tokens, in place."""
@@ -521,8 +557,8 @@ class HipKernels:
         rows, vocab = logits.shape
         self._i32(seq_slot, "seq_slot", rows)
         if logits.dtype != torch.float32 or recent.dtype != torch.int32 or recent_n.dtype != torch.int32 \
-                or recent.dim() != 2 or recent.shape[1] != 64 or not recent.is_contiguous():
-            raise KernelLibraryError("penalty: logits float32, ring int32 [slots, 64], counters int32")
+                or recent.dim() != 2 or recent.shape[1] != self.penalty_window or not recent.is_contiguous():
+            raise KernelLibraryError(f"penalty: logits float32, ring int32 [slots, {self.penalty_window}], counters int32")
         self._check(self.lib.lq_apply_penalty(_ptr(logits), c_int(self._rows2d(logits, "logits")), c_int(rows),
                                               c_int(vocab), _ptr(seq_slot), _ptr(recent), _ptr(recent_n),
                                               c_float(penalty), self.stream))

@@ -113,6 +113,17 @@ class DecoderModel:
                     needs[i] = need
         return needs
 
+    # ---- what a decoding step's launches depend on beside the batch size ---------------
+    def _mixers(self):
+        return [b.mixer for b in self.blocks if getattr(b, "mixer", None) is not None]
+
+    def length_bound(self, kernels, longest: int) -> int:
+        """The largest of the mixers' bounds (`Mixer.length_bound`); `longest` itself without mixers."""
+        return max((m.length_bound(kernels, longest) for m in self._mixers()), default=longest)
+
+    def lengths_uneven(self, kernels, lengths) -> bool:
+        return any(m.lengths_uneven(kernels, lengths) for m in self._mixers())
+
     # ---- one step -------------------------------------------------------------------
     def forward(self, ctx: StepContext, caches: Mapping[int, object], want_rows: torch.Tensor,
                 n_want: int) -> Optional[torch.Tensor]:

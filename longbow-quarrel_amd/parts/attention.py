@@ -67,6 +67,15 @@ class GQAttention(Mixer):
     takes_normed_rows = True
     takes_residual_sink = True
 
+    # the attention kernel's own rules, where the kernel object has them
+    def length_bound(self, kernels, longest: int) -> int:
+        ask = getattr(kernels, "decode_length_bound", None)
+        return ask(longest) if ask is not None else super().length_bound(kernels, longest)
+
+    def lengths_uneven(self, kernels, lengths) -> bool:
+        ask = getattr(kernels, "decode_lengths_uneven", None)
+        return bool(ask(lengths)) if ask is not None and self.window == 0 else False
+
     def forward(self, h, ctx: StepContext, cache: Optional[LayerCache], sink=None) -> Optional[torch.Tensor]:
         if cache is None or cache.k is None:
             raise RuntimeError("attention needs a key/value cache")

@@ -251,7 +251,7 @@ class StepContext:
     max_new: int = 0
     max_len: int = 0
     decode: bool = False  # every sequence brings exactly one token
-    # a decoding step whose sequences differ much in length (`lengths_uneven`): a hint, which changes how the
+    # a decoding step whose sequences differ much in length (`Mixer.lengths_uneven`): a hint, which changes how the
     # attention kernel shares its work out and nothing in the result beyond the order of its sums
     uneven: bool = False
     logits_out: Optional[torch.Tensor] = None  # where the logits go (a captured step's fixed buffer)
@@ -396,6 +396,25 @@ class Mixer(Part):
     def cache_need(self):
         """KVNeed, StateNeed or None."""
         return None
+
+    # What a decoding step's launches depend on beside its batch size.  The engine asks every mixer and
+    # keeps a captured step for as long as the answers stay the same; `ctx.max_len` and `ctx.uneven` carry
+    # them (the largest bound and any yes over the model's mixers) into `forward`.
+    def length_bound(self, kernels, longest: int) -> int:
+        """An upper bound of the sequence lengths for a decoding step whose longest sequence holds
+        `longest` tokens.  Steps with one bound must be the same launches: the coarser the bound, the fewer
+        captured steps.  Default: the next power of two (at least 64), for a mixer whose launches do not
+        depend on the lengths at all or that reads `ctx.max_len` without a rule of its own."""
+        bound = 64
+        while bound < longest:
+            bound *= 2
+        return bound
+
+    def lengths_uneven(self, kernels, lengths) -> bool:
+        """Whether the mixer wants a decoding step with these lengths (after the step) marked `ctx.uneven`:
+        a hint that may change how its launches share out their work and nothing in the result beyond the
+        order of its sums."""
+        return False
 
     def forward(self, h: torch.Tensor, ctx: StepContext, cache: Optional[LayerCache]) -> torch.Tensor:
         raise NotImplementedError

@@ -16,7 +16,13 @@ class NonFiniteLogits(RuntimeError):
     """A row of logits holds a NaN or an infinity.  The reference scans for them and falls back to the
     first finite index (internal/engine/sampler.go:73-75, 107-123); a library that is checked for
     exactness reports the fault instead.  The kernels write `NO_TOKEN` for such a row and leave its
-    generator and its ring of recent ids alone; whoever reads the tokens back raises this."""
+    generator and its ring of recent ids alone; whoever reads the tokens back raises this.  Raised by the
+    generation loop it carries `result`: what every request had got by then, the faulty ones with the finish
+    "error" and the others run to their own ends."""
+
+    def __init__(self, message: str, result=None) -> None:
+        super().__init__(message)
+        self.result = result
 
 
 class Sampler:

@@ -23,11 +23,13 @@ def sequence_key(seed: int, index: int) -> int:
 
 
 class SamplerState:
-    def __init__(self, max_slots: int, device: torch.device) -> None:
+    def __init__(self, max_slots: int, device: torch.device, window: int = RECENT) -> None:
+        """`window`: ids of history that the penalty looks at (the sampling kernels say which width they take)."""
         self.device = device
+        self.window = int(window)
         self.rng_key = torch.zeros(max_slots, dtype=torch.int64, device=device)
         self.rng_ctr = torch.zeros(max_slots, dtype=torch.int64, device=device)
-        self.recent = torch.full((max_slots, RECENT), -1, dtype=torch.int32, device=device)
+        self.recent = torch.full((max_slots, self.window), -1, dtype=torch.int32, device=device)
         self.recent_n = torch.zeros(max_slots, dtype=torch.int32, device=device)
         # what the two stages of the arg-max kernel pass between them: 32 words for each row of a batch
         self.argmax_scratch = torch.zeros(32 * max_slots, dtype=torch.int64, device=device)
@@ -44,13 +46,14 @@ class SamplerState:
 
     def start(self, slot: int, key: int, history: Sequence[int]) -> None:
         """A sequence starts in `slot`: generator at draw 0, ring holding the end of its prompt."""
-        tail = list(history[-RECENT:])
-        row = torch.full((RECENT,), -1, dtype=torch.int32)
+        ring = self.window
+        tail = list(history[-ring:])
+        row = torch.full((ring,), -1, dtype=torch.int32)
         if tail:
-            # the ring is written at n % 64; lay the tail out as if it had been pushed one by one
+            # the ring is written at n % its width; lay the tail out as if it had been pushed one by one
             n = len(history)
             for j, tok in enumerate(tail):
-                row[(n - len(tail) + j) % RECENT] = int(tok)
+                row[(n - len(tail) + j) % ring] = int(tok)
         self.recent[slot].copy_(row)
         self.recent_n[slot : slot + 1].copy_(torch.tensor([len(history)], dtype=torch.int32))
         self.rng_key[slot : slot + 1].copy_(torch.tensor([key], dtype=torch.int64))

@@ -67,5 +67,72 @@ def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
 
 # Tolerances, fixed once: float32 against float64 arithmetic; bfloat16 against the plain
 # implementation that rounds activations to bfloat16 at the same places.
-TOL_F32 = 2e-5
+# Measured on the GPU, float32 engine against the float64 plain implementation, whole prompts of 1 to 400
+# tokens: 2.2e-7 to 7.8e-7 on the tiny configurations with weights of standard deviation 0.02 to 0.1, 3.3e-6
+# with the peaked attention of standard deviation 0.15.  One case is harsher by construction (weights of 0.1,
+# norm gains 1 +- 0.4, head size 144): its worst single row reads 1.3e-5 and keeps the limit that it always
+# had, TOL_F32_HARSH.
+TOL_F32 = 1e-5
+TOL_F32_HARSH = 2e-5
 TOL_BF16 = 1.5e-2
+
+
+def stopping_scenarios(eng, graphs_cls=None):
+    """Two orders of events around a step that is queued ahead, through captured steps against direct ones.
+
+    (1) The cache is as full as it may be (4 blocks).  C holds block 0 and ends on its fourth token; the step
+    queued ahead still ran for C and wrote into block 0.  In the very next step A passes 64 tokens and is
+    handed block 0, the only free one.  (2) Every sequence of a batch ends on a stop id while a step is queued
+    ahead, and the next batch starts on the same slots and blocks."""
+    import longbow_quarrel_amd as lq
+    from longbow_quarrel_amd.engine.generate import EngineBackend, GenerationLoop
+
+    def run(prompts, n, stops, graphs, max_batch=3):
+        kw = {} if graphs_cls is None else {"graphs_cls": graphs_cls}
+        be = EngineBackend(eng, lq.SamplingParams(), use_graphs=graphs, **kw)
+        try:
+            return GenerationLoop(be, max_batch=max_batch).run(prompts, n, stop_ids=stops), be.steps_ahead
+        finally:
+            be.close()
+
+    vocab = eng.vocab_size
+    for seed in range(31, 31 + 3 * 20, 3):  # (the first prompts with which the events fall as the scenario wants)
+        c, a, b = random_tokens(5, vocab, seed), random_tokens(60, vocab, seed + 1), random_tokens(10, vocab, seed + 2)
+        free, _ = run([c, a, b], 10, [], False)
+        stop = free.tokens[0][3]
+        if stop not in free.tokens[0][:3] and stop not in free.tokens[1] and stop not in free.tokens[2]:
+            break
+    else:
+        raise AssertionError("no prompts found whose first request alone meets its stop id")
+    direct, _ = run([c, a, b], 10, [stop], False)
+    assert direct.finish == ["stop", "length", "length"] and len(direct.tokens[0]) == 3
+    table = eng.cache.kv_groups[0]
+    seen = []
+    ensure = table.ensure
+
+    def watch(slot, new_len):
+        before = list(table.owned[slot])
+        ensure(slot, new_len)
+        if len(table.owned[slot]) > len(before) and before:
+            seen.append((new_len, table.owned[slot][len(before):]))
+
+    table.ensure = watch
+    try:
+        got, ahead = run([c, a, b], 10, [stop], True)
+    finally:
+        table.ensure = ensure
+    assert got.tokens == direct.tokens and got.finish == direct.finish and ahead > 0
+    assert seen == [(65, [0])]  # A's 65th token went into the block that C had just given back
+    # (2) all of a batch stop at once, a step is queued, the next batch takes over slots and blocks
+    for seed in range(50, 50 + 7 * 20, 7):
+        prompts = [random_tokens(3 + i, vocab, seed + i) for i in range(6)]
+        free, _ = run(prompts, 8, [], False)
+        stops = sorted({t[2] for t in free.tokens[:3]})
+        direct, _ = run(prompts, 8, stops, False)
+        if direct.finish[:3] == ["stop"] * 3 and direct.batches == 2 and "length" in direct.finish:
+            break
+    else:
+        raise AssertionError("no prompts found whose first batch ends on stop ids alone")
+    got, ahead = run(prompts, 8, stops, True)
+    assert got.tokens == direct.tokens and got.finish == direct.finish and ahead > 0
+    assert eng.cache.slots.taken_count == 0 and eng.cache.free_blocks() == eng.cache.n_blocks

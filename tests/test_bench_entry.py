@@ -36,6 +36,9 @@ def test_bytes_and_flops_of_the_8b_shape_by_hand():
     attention = 2 * 2 * 32 * 128 * t * (t + 1) / 2
     assert bench.prefill_flops(c, t) == pytest.approx(layers * (linear + attention) + 2 * d * v, rel=1e-12)
     assert 2.9e13 < bench.prefill_flops(c, t) < 3.1e13
+    # the 32-bit path: every matrix and the cache at four bytes an entry, the norms' gains as before
+    assert bench.weight_bytes_per_step(c, 4) == layers * (2 * per_layer - 2 * 4 * d) + 4 * v * d + 4 * d
+    assert bench.kv_bytes_per_token(c, 4) == 2 * 131072
 
 
 def test_the_other_shapes_are_the_family_s_sizes():

@@ -8,13 +8,13 @@ import longbow_quarrel_amd as lq
 import plain
 import toy_parts
 from cpu_kernels import CpuKernels
-from helpers import TINY_A, TINY_B, TINY_C, random_tokens, read_folder, rel_err, write_folder
+from helpers import TINY_A, TINY_B, TINY_C, random_tokens, read_folder, rel_err, stopping_scenarios, write_folder
 from longbow_quarrel_amd.cache import CacheFull
 from longbow_quarrel_amd.engine import StepEntry
 from longbow_quarrel_amd.loading import random_engine
 from longbow_quarrel_amd.weights import random_tensors
 
-TOL = 2e-5
+TOL = 1e-5
 
 
 def make(tmp_path, cfg, seed=7, max_tokens=1024, max_sequence_tokens=4096):
@@ -257,6 +257,12 @@ def test_steps_queued_ahead_give_the_same_tokens_and_none_is_wasted_at_a_known_e
         assert be.ahead is None and eng.cache.slots.taken_count == 0
 
 
+def test_a_freed_block_goes_to_a_survivor_while_a_step_is_queued_and_a_batch_follows_one_that_stopped(tmp_path):
+    eng, ref = make(tmp_path, TINY_A, max_tokens=256)
+    graphs_cls, log = _replayed_graphs()
+    stopping_scenarios(eng, graphs_cls)
+
+
 def test_prompts_run_in_portions_of_at_most_max_prefill_rows(tmp_path):
     """A batch's prompts are fed in steps of a bounded number of rows: several sequences a step, a long
     prompt over several steps (cut at 2 tokens, at a cache block's edge, anywhere), logits only from each
@@ -318,9 +324,30 @@ def test_non_finite_logits_are_reported_not_sampled(tmp_path):
     eng = lq.load_engine(folder, dtype="float32", max_tokens=512, device="cpu", kernels=CpuKernels())
     assert lq.generate(eng, [[1, 2, 3], [4, 5]], 3, stop_ids=[], use_graphs=False).finish == ["length"] * 2
     eng.model.head[17, :] = float("inf")  # token 17's logit overflows for every row
-    with pytest.raises(lq.NonFiniteLogits, match="request 0"):
+    with pytest.raises(lq.NonFiniteLogits, match="request 0") as caught:
         lq.generate(eng, [[1, 2, 3], [4, 5]], 3, stop_ids=[], use_graphs=False)
+    assert caught.value.result.finish == ["error", "error"] and caught.value.result.tokens == [[], []]
     assert eng.cache.slots.taken_count == 0  # the failed call gave its slots back
+
+
+def test_one_faulty_request_ends_alone_and_the_others_keep_their_tokens(tmp_path):
+    """Only the request whose logits are not finite ends (finish "error"); the others of its batch and the
+    batch after it run to their ends with the tokens they get without it, and the error that is raised at the
+    end carries all of them."""
+    folder = write_folder(tmp_path, TINY_A, 5, dtype=torch.float32)
+    eng = lq.load_engine(folder, dtype="float32", max_tokens=512, device="cpu", kernels=CpuKernels())
+    prompts = [[1, 2, 3], [4, 5], [9, 8, 7, 6], [11]]
+    good = lq.generate(eng, prompts, 4, stop_ids=[], use_graphs=False, max_batch=3)
+    # request 1 alone goes wrong, from its second token on: the embedding row of its first token is not finite
+    first = good.tokens[1][0]
+    assert all(first not in t for i, t in enumerate(good.tokens) if i != 1) and first not in sum(prompts, [])
+    eng.model.embedding.table[first, 0] = float("nan")
+    with pytest.raises(lq.NonFiniteLogits, match=r"request 1 \(slot") as caught:
+        lq.generate(eng, prompts, 4, stop_ids=[], use_graphs=False, max_batch=3)
+    res = caught.value.result
+    assert res.finish == ["length", "error", "length", "length"] and res.batches == 2
+    assert res.tokens == [good.tokens[0], [first], good.tokens[2], good.tokens[3]]
+    assert eng.cache.slots.taken_count == 0
 
 
 def test_workspace_lifetimes():

@@ -9,10 +9,11 @@ import sys
 import pytest
 import torch
 
+import helpers
 import longbow_quarrel_amd as lq
 import plain
 import toy_parts
-from helpers import TINY_A, TINY_B, TINY_C, TOL_BF16, TOL_F32, random_tokens, read_folder, rel_err, write_folder
+from helpers import TINY_A, TINY_B, TINY_C, TOL_BF16, TOL_F32, TOL_F32_HARSH, random_tokens, read_folder, rel_err, write_folder
 from longbow_quarrel_amd.engine import StepEntry
 from longbow_quarrel_amd.loading import random_engine
 from longbow_quarrel_amd.weights import random_tensors
@@ -214,6 +215,16 @@ def test_steps_queued_ahead_of_the_host_and_a_sequence_that_stops_in_between(tmp
             assert (be.steps_ahead > 0) == ahead
             be.close()
     assert eng.cache.slots.taken_count == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_freed_block_goes_to_a_survivor_while_a_step_is_queued_and_a_batch_follows_one_that_stopped(
+        tmp_path_factory, dtype):
+    """With real captured graphs and a stream that runs behind the host: the orders of events that
+    `helpers.stopping_scenarios` sets up, against direct steps."""
+    folder = write_folder(tmp_path_factory.mktemp("stopping"), TINY_A, seed=7)
+    eng = lq.load_engine(folder, dtype=dtype, max_tokens=256, max_sequence_tokens=4096)
+    helpers.stopping_scenarios(eng)
 
 
 @pytest.mark.parametrize("n_prompts,max_batch", [(6, 3), (2, 1)])
@@ -496,15 +507,16 @@ def test_generation_with_sequences_of_very_unequal_lengths(tmp_path_factory):
     alike (the tokens and the logits of both are equal), the logits agree with the plain implementation, and
     once the long sequence has ended the rest goes on without the hint."""
     from longbow_quarrel_amd.engine.generate import EngineBackend, GenerationLoop
-    from longbow_quarrel_amd.engine.step import lengths_uneven
 
-    assert lengths_uneven([1401, 61, 26, 301]) and not lengths_uneven([530] * 8) and not lengths_uneven([900])
-    assert not lengths_uneven([1000, 985, 300]) and lengths_uneven([3000, 1000])
     folder = write_folder(tmp_path_factory.mktemp("uneven"), LONG, seed=10, std=0.08)
     c, tensors = read_folder(folder)
     ref = plain.PlainLlama(c, tensors)
     eng = lq.load_engine(folder, dtype="bfloat16", max_tokens=4096)
     kn = eng.kernels
+    lengths_uneven = eng.lengths_uneven  # the engine asks the model, the model its mixers, they the kernel object
+    assert lengths_uneven([1401, 61, 26, 301]) and not lengths_uneven([530] * 8) and not lengths_uneven([900])
+    assert not lengths_uneven([1000, 985, 300]) and lengths_uneven([3000, 1000])
+    assert eng.length_bound(1) == eng.length_bound(1024) == 1024 and eng.length_bound(1025) == 2048
     prompts = [random_tokens(n, LONG["vocab_size"], 800 + n) for n in (300, 290, 310, 1400)]
     hints = []
     attention = kn.attention
@@ -601,7 +613,7 @@ def test_large_weights_on_the_size_agnostic_attention_kernel(tmp_path_factory):
     def worst_row(a, b):
         return max(rel_err(a[i], b[i]) for i in range(len(toks)))
 
-    assert worst_row(replay("float32"), exact) < TOL_F32
+    assert worst_row(replay("float32"), exact) < TOL_F32_HARSH
     got = replay("bfloat16")
     noise = worst_row(moved, rounded)
     assert 1e-2 < noise < 1e-1  # what this test is about: the model's own noise is above the fixed bound
@@ -650,6 +662,23 @@ def test_command_line_generates_the_same_greedy_tokens(tmp_path_factory):
     assert out.returncode == 0, out.stderr[-2000:]
     assert out.stdout.strip().splitlines()[-1].split() == [str(t) for t in expect[:cut]]
     assert f"{cut} tokens in" in out.stdout
+    # prompts from a file (two requests, one batch), the other spelling of the token count, and a stop id of
+    # the caller's: request 0 ends before the token it would have produced third
+    other = reqs[0]
+    both = lq.generate(eng, [prompt, other], 6, stop_ids=[]).tokens
+    stop = both[0][2]
+    expect2 = lq.generate(eng, [prompt, other], 6, extra_stop_ids=[stop]).tokens
+    assert len(expect2[0]) <= 2
+    path = os.path.join(folder, "prompts.txt")
+    with open(path, "w") as f:
+        f.write(" ".join(map(str, prompt)) + "\n\n" + ",".join(map(str, other)) + "\n")
+    out = subprocess.run([sys.executable, os.path.join(root, "bin", "quarrel"), "-model", folder, "-prompt-file", path,
+                          "-max-new-tokens", "6", "-stop-id", str(stop), "-temp", "0", "-penalty", "1",
+                          "-dtype", "float32"], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = out.stdout.strip().splitlines()[-2:]
+    assert [line.split()[1:] for line in lines] == [[str(t) for t in ids] for ids in expect2]
+    assert [line.split()[0] for line in lines] == ["[0]", "[1]"]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -149,9 +149,19 @@ def test_sampling_params_and_sequence_keys():
 
 
 def test_when_a_step_calls_its_lengths_uneven():
-    """The hint to the attention kernel is a function of the lengths alone: the longest at least half again the
-    mean, two sequences or more, and something to share out (512 tokens)."""
-    from longbow_quarrel_amd.engine.step import lengths_uneven
+    """The hint to the attention kernel is the kernel library's own function of the lengths alone (a host
+    function, callable without a GPU): the longest at least half again the mean, two sequences or more, and
+    something to share out (512 tokens).  The bound of the lengths is the longest rounded up to the library's
+    bucket.  The engine asks its model, the model its mixers, and a mixer without a rule gives a power of two."""
+    import ctypes
+
+    from longbow_quarrel_amd import build
+    from longbow_quarrel_amd.parts.base import Mixer
+
+    lib = ctypes.CDLL(build.ensure_built())
+
+    def lengths_uneven(lengths):
+        return bool(lib.lq_attention_lengths_uneven((ctypes.c_int * max(1, len(lengths)))(*lengths), len(lengths)))
 
     assert lengths_uneven([3000, 1000]) and lengths_uneven([1401, 61, 26, 301]) and lengths_uneven([600, 200, 100])
     assert not lengths_uneven([530] * 8) and not lengths_uneven([4000]) and not lengths_uneven([])
@@ -159,3 +169,26 @@ def test_when_a_step_calls_its_lengths_uneven():
     assert not lengths_uneven([500, 20, 30])         # nothing long enough to share out
     assert lengths_uneven([1500, 1000, 500]) and not lengths_uneven([1499, 1000, 501])  # the bound itself: 1.5
     assert lengths_uneven([5000] + [4000] * 63) is False and lengths_uneven([8000] + [100] * 63)
+    assert lib.lq_attention_length_bucket() > 0 and lib.lq_attention_length_bucket() % 64 == 0
+    plain_mixer = Mixer()
+    assert [plain_mixer.length_bound(None, n) for n in (1, 64, 65, 1000, 1025)] == [64, 64, 128, 1024, 2048]
+    assert plain_mixer.lengths_uneven(None, [3000, 1000]) is False
+
+
+def test_command_line_options_have_the_reference_names_and_a_few_more():
+    """cmd/quarrel/main_metal.go:24-36 and cmd/generate_text/main.go:18-26 name the options; the count of
+    tokens also answers to -len and -max-new-tokens, stop ids may be given several times."""
+    from longbow_quarrel_amd.cli import build_parser
+
+    ap = build_parser()
+    a = ap.parse_args(["-model", "m", "-prompt", "1 2", "-n", "7", "-kv-cache-size", "99", "-temp", "0.5", "-topk", "3",
+                       "-topp", "0.9", "-penalty", "1.2", "-stream"])
+    assert (a.model, a.prompt, a.n, a.kv_cache_size, a.temp, a.topk, a.topp, a.penalty, a.stream) == \
+        ("m", "1 2", 7, 99, 0.5, 3, 0.9, 1.2, True)
+    d = ap.parse_args(["-model", "m"])
+    assert (d.prompt_file, d.prompt_ids, d.stop_ids, d.n, d.kv_cache_size, d.temp, d.topk, d.topp, d.penalty) == \
+        ("", "", [], 20, 2048, 0.7, 40, 0.95, 1.1)
+    for spelling in ("-len", "--len", "-max-new-tokens", "--max-new-tokens", "--n"):
+        assert ap.parse_args(["-model", "m", spelling, "5"]).n == 5
+    b = ap.parse_args(["--model", "m", "--stop-id", "4", "-stop-id", "9", "--prompt-file", "p.txt", "--prompt-ids", "1,2"])
+    assert b.stop_ids == [4, 9] and b.prompt_file == "p.txt" and b.prompt_ids == "1,2"
