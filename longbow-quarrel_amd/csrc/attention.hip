@@ -1,7 +1,7 @@
 // lq_attention: causal grouped-query attention over the paged cache, dispatch.
 #include "common.h"
 
-int lq_attention_generic(const void* q, int ldq, void* out, int ldo, int dtype, int rows, int nh,
+int lq_attention_generic(const void* q, int ldq, void* out, int ldo, int dtype, int rows, int batch, int nh,
                          int nkv, int hd, const int* row_pos, const int* row_seq,
                          const int* seq_slot, const int* block_table, int bt_stride,
                          const void* kcache, const void* vcache, int block_size, float scale,
@@ -87,6 +87,6 @@ extern "C" int lq_attention(const void* q, int ldq, void* out, int ldo, int dtyp
                              workspace, workspace_floats, tickets, tickets_n, k_new, v_new, ldk, ldv, cs, uneven,
                              pieces, piece_stride, stream);
   LQ_REQUIRE(cs == nullptr && pieces <= 1, "attention: the folded rotation was asked of a launch the matrix-core kernel does not take");
-  return lq_attention_generic(q, ldq, out, ldo, dtype, rows, nh, nkv, hd, row_pos, row_seq, seq_slot,
+  return lq_attention_generic(q, ldq, out, ldo, dtype, rows, batch, nh, nkv, hd, row_pos, row_seq, seq_slot,
                               block_table, bt_stride, kcache, vcache, block_size, scale, window, stream);
 }
