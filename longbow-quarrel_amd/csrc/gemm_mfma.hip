@@ -710,9 +710,12 @@ __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16
                                                                       long long split_stride, RowScale scale,
                                                                       ResidualOut res) {
   constexpr int KB = v3_kb(MT);
-  constexpr int NBUF = MT == 1 ? 2 : 1;
   constexpr int VALS = MT * 4;  // accumulator values a lane holds per tile
-  __shared__ float red[NBUF][KW][VALS * 64];
+  // One row tile: the partial tiles of all the block's column tiles meet in LDS at once (dynamic, a KiB a tile
+  // and wave), behind one barrier.  More row tiles: a tile at a time through a buffer of fixed size.
+  constexpr bool BATCH = MT == 1;
+  __shared__ float red_one[BATCH ? 1 : KW][BATCH ? 1 : VALS * 64];
+  extern __shared__ __attribute__((aligned(16))) float red_all[];  // [tiles][KW][256] with BATCH
   __shared__ float fresh_sh[EPI == EPI_RESIDUAL ? 16 : 1][EPI == EPI_RESIDUAL ? V3_MAXT * 16 : 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, c16 = lane & 15;
@@ -787,44 +790,82 @@ __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16
       for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
       if (lane == 0) rstd_sh[wave] = 1.0f / sqrtf(sum / (float)scale.width + scale.eps);
     }
-    // the barrier of the first tile's reduction below also publishes rstd_sh
+    // the barrier of the reduction below also publishes rstd_sh
   }
   // acc[t][m][e] = C[m * 16 + (lane / 16) * 4 + e][col_begin + 16 t + lane % 16], partial over this
-  // wave's k.  The waves share out the (m, e) values of a tile and each sums its share over all waves,
+  // wave's k.  The waves share out the (m, e) values of the tiles and each sums its share over all waves,
   // in wave order.
+  auto finish = [&](int t, int v, float s, float x_old) {
+    const int col = col_begin + t * 16 + c16;
+    const int row = (v >> 2) * 16 + g * 4 + (v & 3);
+    if (SCALED) s *= rstd_sh[min(row, M - 1)];
+    if (EPI == EPI_SWIGLU) {
+      const float up = __shfl(s, lane + 8, 64);
+      if (c16 < 8 && row < M && col + 8 < col_end)
+        store_out<TO>(C + (long long)row * ldc + ((col_begin + t * 16) >> 1) + c16, silu_mul(s, up));
+    } else if constexpr (EPI == EPI_RESIDUAL) {
+      static_assert(EPI != EPI_RESIDUAL || sizeof(TO) == 4, "the residual stream is float32");
+      float fresh = 0.f;
+      if (row < M && col < col_end) {
+        fresh = x_old + s;
+        *((float*)C + (long long)row * ldc + col) = fresh;
+        if (res.scaled) res.scaled[(long long)row * res.ld_scaled + col] = f32_to_bf16(fresh * res.gain[col]);
+      }
+      if (row < 16) fresh_sh[row][t * 16 + c16] = fresh;  // zero beyond the matrix
+    } else {
+      if (row < M && col < col_end) store_out<TO>(C + (long long)row * ldc + col, s);
+    }
+  };
+  auto stream_value = [&](int t, int v) -> float {  // the residual stream's old value at this lane's place
+    if constexpr (EPI == EPI_RESIDUAL) {
+      const int col = col_begin + t * 16 + c16, row = (v >> 2) * 16 + g * 4 + (v & 3);
+      if (row < M && col < col_end) return *((const float*)C + (long long)row * ldc + col);
+    }
+    return 0.f;
+  };
+  if constexpr (BATCH) {
+    // every tile's partial sums at once; the 4 value rows of each tile are dealt out over the waves (row
+    // j = 4 t + v to wave j % KW), which ask for the stream's old values before they meet at the barrier
+    static_assert(!BATCH || V3_MAXT * 4 <= 2 * KW, "at most two value rows a wave");
 #pragma unroll
-  for (int t = 0; t < V3_MAXT; ++t) {
-    if (t < ntiles) {
-      float(*r)[VALS * 64] = red[NBUF == 2 ? (t & 1) : 0];
-      if (NBUF == 1 && t > 0) __syncthreads();  // the tile before has been read
+    for (int t = 0; t < V3_MAXT; ++t)
+      if (t < ntiles) {
 #pragma unroll
-      for (int m = 0; m < MT; ++m)
+        for (int e = 0; e < 4; ++e) red_all[(t * KW + wave) * 256 + e * 64 + lane] = acc[t][0][e];
+      }
+    float x_old[2];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) r[wave][(m * 4 + e) * 64 + lane] = acc[t][m][e];
-      __syncthreads();  // with two buffers also: the buffer written two tiles ago has been read by then
-      const int col = col_begin + t * 16 + c16;
-      for (int v = (wave + t) % KW; v < VALS; v += KW) {
+    for (int i = 0; i < 2; ++i) {
+      const int j = wave + KW * i;
+      x_old[i] = j < ntiles * 4 ? stream_value(j >> 2, j & 3) : 0.f;
+    }
+    __syncthreads();  // (also publishes rstd_sh)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int j = wave + KW * i;
+      if (j < ntiles * 4) {
+        const int t = j >> 2, v = j & 3;
         float s = 0.f;
 #pragma unroll
-        for (int w = 0; w < KW; ++w) s += r[w][v * 64 + lane];
-        const int row = (v >> 2) * 16 + g * 4 + (v & 3);
-        if (SCALED) s *= rstd_sh[min(row, M - 1)];
-        if (EPI == EPI_SWIGLU) {
-          const float up = __shfl(s, lane + 8, 64);
-          if (c16 < 8 && row < M && col + 8 < col_end)
-            store_out<TO>(C + (long long)row * ldc + ((col_begin + t * 16) >> 1) + c16, silu_mul(s, up));
-        } else if constexpr (EPI == EPI_RESIDUAL) {
-          static_assert(EPI != EPI_RESIDUAL || sizeof(TO) == 4, "the residual stream is float32");
-          float fresh = 0.f;
-          float* xr = (float*)C + (long long)row * ldc + col;
-          if (row < M && col < col_end) {
-            fresh = *xr + s;
-            *xr = fresh;
-            if (res.scaled) res.scaled[(long long)row * res.ld_scaled + col] = f32_to_bf16(fresh * res.gain[col]);
-          }
-          if (row < 16) fresh_sh[row][t * 16 + c16] = fresh;  // zero beyond the matrix
-        } else {
-          if (row < M && col < col_end) store_out<TO>(C + (long long)row * ldc + col, s);
+        for (int w = 0; w < KW; ++w) s += red_all[(t * KW + w) * 256 + v * 64 + lane];
+        finish(t, v, s, x_old[i]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < V3_MAXT; ++t) {
+      if (t < ntiles) {
+        if (t > 0) __syncthreads();  // the tile before has been read
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) red_one[wave][(m * 4 + e) * 64 + lane] = acc[t][m][e];
+        __syncthreads();
+        for (int v = (wave + t) % KW; v < VALS; v += KW) {
+          float s = 0.f;
+#pragma unroll
+          for (int w = 0; w < KW; ++w) s += red_one[w][v * 64 + lane];
+          finish(t, v, s, stream_value(t, v));
         }
       }
     }
@@ -875,7 +916,19 @@ int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K,
   v3_runs(N, lq_compute_units() / splits, EPI == EPI_SWIGLU ? 16 : 8, cols, grid);
   const int ksteps = lq_ceil_div(K, 32);
   const int ks_per_wave = lq_ceil_div(ksteps, KW * splits);
-  gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO, SCALED><<<dim3(grid, splits), KW * 64, 0, stream>>>(
+  auto kernel = gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO, SCALED>;
+  // one row tile: a KiB of LDS for every column tile and wave of a block
+  const int lds = MT == 1 ? lq_ceil_div(cols, 16) * KW * 1024 : 0;
+  static bool configured = false;
+  if (!configured && MT == 1) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, V3_MAXT * KW * 1024);
+    if (e != hipSuccess) {
+      lq_set_error("linear: cannot reserve %d bytes of LDS: %s", V3_MAXT * KW * 1024, hipGetErrorString(e));
+      return -2;
+    }
+    configured = true;
+  }
+  kernel<<<dim3(grid, splits), KW * 64, lds, stream>>>(
       (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, cols, ks_per_wave, split_stride, scale, res);
   LQ_CHECK_LAUNCH("linear(mfma skinny v3)");
   return 0;

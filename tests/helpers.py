@@ -9,7 +9,6 @@ from typing import Dict, List, Sequence
 import torch
 
 import longbow_quarrel_amd as lq
-from longbow_quarrel_amd.weights.safetensors_io import SafetensorsFile
 
 # Two tiny Llama configurations that share no size or option.
 TINY_A = {
@@ -47,9 +46,11 @@ def write_folder(tmp_path, cfg: Dict, seed: int, dtype=None, std: float = 0.02) 
 def read_folder(folder: str):
     with open(os.path.join(folder, "config.json")) as f:
         cfg = json.load(f)
-    sf = SafetensorsFile(os.path.join(folder, "model.safetensors"))
-    tensors = {n: sf.tensor(n) for n in sf.names()}
-    sf.close()
+    # read with the container format's own package, not with the library's reader: a fault of that reader
+    # (an offset, a byte order) must not reach the plain implementation and the engine alike
+    from safetensors.torch import load_file
+
+    tensors = load_file(os.path.join(folder, "model.safetensors"))
     return cfg, tensors
 
 

@@ -407,6 +407,54 @@ def test_decoding_batches_that_shrink_from_40_rows_to_one(tmp_path_factory):
     assert any(r > 32 for r in in_pieces) and any(16 < r <= 32 for r in in_pieces) and not any(r <= 16 for r in in_pieces)
 
 
+def test_the_float32_path_at_the_width_of_a_real_model(tmp_path_factory):
+    """One layer with the 8B shape's width, heads and head size (4 096 wide, 32 heads over 8 of 128; the inner width and
+    the vocabulary no powers of two) in true float32: whole prompts of 1 to 150 tokens against the float64 plain
+    implementation (the K of the products is 4 096 and 5 000 here, where the tiny configurations end at 520), and a
+    request fed whole, with its last tokens one by one, and inside a batch of unequal lengths gives the same bits."""
+    cfg = {
+        "architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "intermediate_size": 5000,
+        "num_hidden_layers": 1, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+        "vocab_size": 1031, "max_position_embeddings": 512, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+        "rope_scaling": None, "tie_word_embeddings": False, "torch_dtype": "float32", "bos_token_id": 1, "eos_token_id": 2,
+    }
+    folder = write_folder(tmp_path_factory.mktemp("wide32"), cfg, seed=12, std=0.02)
+    c, tensors = read_folder(folder)
+    ref = plain.PlainLlama(c, tensors)
+    eng = lq.load_engine(folder, dtype="float32", max_tokens=1024)
+    reqs = [random_tokens(n, cfg["vocab_size"], 900 + n) for n in (150, 1, 40, 17)]
+    whole = []
+    for r in reqs:
+        s = eng.new_sequence()
+        whole.append(eng.step([StepEntry(s, r, range(len(r)))]))
+        eng.release(s)
+        assert rel_err(whole[-1], ref.forward(r)) < TOL_F32, len(r)
+    # the last 20 tokens of the first request one by one
+    s = eng.new_sequence()
+    got = [eng.step([StepEntry(s, reqs[0][:130], range(130))])]
+    got += [eng.step([StepEntry(s, [t], [0])]) for t in reqs[0][130:]]
+    eng.release(s)
+    assert torch.equal(torch.cat(got), whole[0])
+    # all four in one batch, cut at other places, the shorter ones ending earlier
+    slots = [eng.new_sequence() for _ in reqs]
+    cuts = [100, 1, 33, 16]
+    out = eng.step([StepEntry(sl, r[:n], range(n)) for sl, r, n in zip(slots, reqs, cuts)])
+    at = 0
+    for i, n in enumerate(cuts):
+        assert torch.equal(out[at : at + n], whole[i][:n]), i
+        at += n
+    pos = list(cuts)
+    while any(p < len(r) for p, r in zip(pos, reqs)):
+        live = [i for i, r in enumerate(reqs) if pos[i] < len(r)]
+        out = eng.step([StepEntry(slots[i], [reqs[i][pos[i]]], [0]) for i in live])
+        for j, i in enumerate(live):
+            assert torch.equal(out[j], whole[i][pos[i]]), (i, pos[i])
+            pos[i] += 1
+    for sl in slots:
+        eng.release(sl)
+    assert eng.cache.slots.taken_count == 0
+
+
 LONG = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermediate_size": 264,
     "num_hidden_layers": 2, "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 128,

@@ -101,13 +101,39 @@ def test_swiglu(kn, out_dtype):
 
 # --------------------------------------------------------------------------- linear
 
-@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (5, 331, 80), (70, 130, 333), (129, 65, 17), (3, 1000, 4096)])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (5, 331, 80), (70, 130, 333), (129, 65, 17), (3, 1000, 4096),
+                                   (16, 4096, 4096), (8, 1000, 14336), (2, 50, 260), (300, 700, 1000), (64, 4096, 520)])
 def test_linear_float32(kn, m, n, k):
     x, w = rnd((m, k), 10), rnd((n, k), 11)
     out = torch.empty((m, n), dtype=torch.float32, device=DEV)
     kn.linear(x, w, out)
     want = x.double().cpu() @ w.double().cpu().t()
     assert rel_err(out, want) < 2e-6
+
+
+@pytest.mark.parametrize("n,k", [(700, 4096), (4100, 1000), (130, 14336), (64, 255)])
+def test_linear_float32_gives_a_row_the_same_bits_in_every_launch(kn, n, k):
+    """The float32 product has three shapes of launch (up to 16 rows streamed from memory with K shared over a
+    block's waves, tiles of 64 x 64, tiles of 128 x 128) and one summation tree: a row comes out bit for bit the
+    same alone, among 9, among 40 and among 300 rows, from dense rows and from a view with a stride."""
+    x, w = rnd((300, k), 20), rnd((n, k), 21)
+    whole = torch.empty((300, n), dtype=torch.float32, device=DEV)
+    kn.linear(x, w, whole)
+    assert rel_err(whole, x.double().cpu() @ w.double().cpu().t()) < 2e-6
+    for rows in (1, 9, 16, 17, 40, 64, 65):
+        part = torch.empty((rows, n), dtype=torch.float32, device=DEV)
+        kn.linear(x[:rows], w, part)
+        assert torch.equal(part, whole[:rows]), rows
+    wide = torch.zeros((9, k + 4), dtype=torch.float32, device=DEV)  # rows 16 bytes further apart than they are long
+    wide[:, :k] = x[100:109]
+    part = torch.empty((9, n), dtype=torch.float32, device=DEV)
+    kn.linear(wide[:, :k], w, part)
+    assert torch.equal(part, whole[100:109])
+    if k % 4 == 0:
+        odd = torch.zeros((9, k + 1), dtype=torch.float32, device=DEV)  # rows that do not start at 16-byte addresses
+        odd[:, :k] = x[100:109]
+        kn.linear(odd[:, :k], w, part)
+        assert torch.equal(part, whole[100:109])
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
@@ -283,14 +309,19 @@ def paged_cache(lengths, kv_heads, head_dim, dtype, seed):
 
 
 def run_attention(kn, q_rows, lengths, new, heads, kv_heads, head_dim, dtype, seed, window=0, decode=False,
-                  force_generic=False, standout=None, max_len=None, uneven=False, check=None):
+                  force_generic=False, standout=None, max_len=None, uneven=False, check=None, q_by_position=False):
     """q rows for the last `new[b]` positions of each sequence; returns (got, want).  With `check` (rows of
     the step, counted through all sequences) only these rows are worked out by the plain implementation
-    and returned: for steps of thousands of rows."""
+    and returned: for steps of thousands of rows.  With `q_by_position` the query of a position of a sequence is
+    the same whatever rows the step brings (for comparisons between steps)."""
     kc, vc, table, slots, dense = paged_cache(lengths, kv_heads, head_dim, dtype, seed)
     g = torch.Generator().manual_seed(seed + 1)
     rows = sum(new)
     q = torch.randn((rows, heads * head_dim), generator=g).to(dtype)
+    if q_by_position:
+        per_seq = [torch.randn((n, heads * head_dim), generator=torch.Generator().manual_seed(seed + 7 + b)).to(dtype)
+                   for b, n in enumerate(lengths)]
+        q = torch.cat([qs[n - m:] for qs, n, m in zip(per_seq, lengths, new)])
     if standout is not None:
         # one far key that every query must find: its score stands out by construction
         b, t = standout
@@ -490,6 +521,29 @@ def test_attention_with_eight_query_heads_a_kv_head(kn, heads, kv_heads):
         check = [0, 31, 32, 1000, 3071, 3072, 3098, 3099]
         got, want = run_attention(kn, None, [3100], [3100], heads, kv_heads, 128, torch.bfloat16, 99, check=check)
         assert rel_err(got, want) < 8e-3
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,window", [(4, 2, 64, 0), (6, 3, 48, 0), (8, 2, 128, 0), (3, 1, 144, 0),
+                                                            (4, 2, 16, 0), (4, 4, 32, 70), (5, 1, 20, 0)])
+def test_float32_attention_gives_a_row_the_same_bits_in_every_step(kn, heads, kv_heads, head_dim, window):
+    """The size-agnostic attention (the whole of the float32 path) works on tiles of 16 rows in prompt steps and
+    on single rows in steps of single tokens (head size 20: the kernel with a wavefront a row in both): a row's
+    output is the same bits as the last row of a prompt, alone in a decoding step, and in a decoding step among
+    other sequences; and right against the plain implementation."""
+    lengths = [150, 37, 64, 200]
+    whole, want = run_attention(kn, None, lengths, lengths, heads, kv_heads, head_dim, torch.float32, 71, window=window,
+                                force_generic=True, q_by_position=True)
+    assert rel_err(whole, want) < 2e-6
+    last = [sum(lengths[: b + 1]) - 1 for b in range(len(lengths))]
+    tail, _ = run_attention(kn, None, lengths, [40, 1, 17, 3], heads, kv_heads, head_dim, torch.float32, 71, window=window,
+                            force_generic=True, q_by_position=True)
+    ends = [39, 40, 57, 60]
+    for b in range(len(lengths)):
+        assert torch.equal(tail[ends[b]], whole[last[b]]), b
+    single, _ = run_attention(kn, None, lengths, [1] * 4, heads, kv_heads, head_dim, torch.float32, 71, window=window,
+                              decode=True, force_generic=True, q_by_position=True)
+    for b in range(len(lengths)):
+        assert torch.equal(single[b], whole[last[b]]), b
 
 
 def test_attention_reference_vectors(kn):
