@@ -92,6 +92,9 @@ def main() -> int:
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (the headline run is 8b)")
     ap.add_argument("--no-points", action="store_true", help="skip the prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true", help="run the prefill alone, twice (for profiling)")
+    ap.add_argument("--profile", action="store_true",
+                    help="device time by operation (HIP events around every kernel call): one prefill of "
+                         "--prefill-tokens tokens and --steps direct decoding steps at --batch; prints a table and exits")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="prompt length of --prefill-only (the reported prefill is always of 2,048 tokens)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
@@ -163,6 +166,43 @@ def main() -> int:
         backend.close()
         return batch * steps / dt, dt / steps * 1e3, ctx_mean
 
+    if args.profile:
+        from longbow_quarrel_amd.kernels.timed import TimedKernels
+
+        timed = TimedKernels(engine.kernels)
+        engine.kernels = timed
+
+        def show(title, wall_ms):
+            rows = timed.report()
+            total = sum(ms for _, ms in rows.values())
+            print(f"[profile] {title}: {wall_ms:.3f} ms on the host's clock, {total:.3f} ms inside event pairs", file=sys.stderr)
+            for op, (calls, ms) in rows.items():
+                print(f"[profile]   {ms / total * 100:5.1f}%  {calls:5d} calls  {ms / calls * 1e3:9.1f} us  {op}", file=sys.stderr)
+            timed.reset()
+
+        n = args.prefill_tokens
+        slots = [engine.new_sequence() for _ in range(args.batch)]
+        engine.step([StepEntry(slots[0], random_prompt(n), [n - 1])])  # first launches
+        engine.release(slots[0])
+        slots[0] = engine.new_sequence()
+        timed.reset()
+        t = time.perf_counter()
+        engine.step([StepEntry(slots[0], random_prompt(n), [n - 1])])
+        torch.cuda.synchronize()
+        show(f"prefill of {n} tokens", (time.perf_counter() - t) * 1e3)
+        engine.release(slots[0])
+        slots[0] = engine.new_sequence()
+        engine.step([StepEntry(s, random_prompt(args.prompt_len), [args.prompt_len - 1]) for s in slots])
+        for _ in range(2):
+            engine.step([StepEntry(s, [1], [0]) for s in slots])
+        timed.reset()
+        t = time.perf_counter()
+        for _ in range(args.steps):
+            engine.step([StepEntry(s, [1], [0]) for s in slots])
+        torch.cuda.synchronize()
+        show(f"{args.steps} direct decoding steps at batch {args.batch} (no sampling, not captured)",
+             (time.perf_counter() - t) * 1e3)
+        return 0
     if args.prefill_only:
         n = args.prefill_tokens
         slot = engine.new_sequence()

@@ -407,6 +407,37 @@ def test_decoding_batches_that_shrink_from_40_rows_to_one(tmp_path_factory):
     assert any(r > 32 for r in in_pieces) and any(16 < r <= 32 for r in in_pieces) and not any(r <= 16 for r in in_pieces)
 
 
+def test_device_time_by_operation_with_events_around_every_kernel_call(tmp_path_factory):
+    """`TimedKernels` stands in for the kernel object of an engine: the same logits, and a report that names
+    every operation a step launched with its calls and a positive time (the products by their sizes)."""
+    from longbow_quarrel_amd.kernels.timed import TimedKernels
+
+    eng, ref, act, reqs, want, _ = setup_case(tmp_path_factory, "b", "bfloat16")
+    r = reqs[0]
+    s = eng.new_sequence()
+    plain_run = eng.step([StepEntry(s, r, range(len(r)))])
+    eng.release(s)
+    real = eng.kernels
+    timed = TimedKernels(real)
+    eng.kernels = timed
+    try:
+        s = eng.new_sequence()
+        got = eng.step([StepEntry(s, r, range(len(r)))])
+        eng.step([StepEntry(s, [3], [0])])
+        eng.release(s)
+        report = timed.report()
+    finally:
+        eng.kernels = real
+    assert torch.equal(got, plain_run)
+    layers = TINY_B["num_hidden_layers"]
+    assert report["attention"][0] == 2 * layers and report["embed"][0] == 2
+    products = [k for k in report if k.startswith("linear")]
+    assert any(k.endswith(f"x {TINY_B['vocab_size']} x {TINY_B['hidden_size']}") for k in products)  # the head
+    assert all(calls > 0 and ms > 0 for calls, ms in report.values())
+    timed.reset()
+    assert timed.report() == {}
+
+
 def test_the_float32_path_at_the_width_of_a_real_model(tmp_path_factory):
     """One layer with the 8B shape's width, heads and head size (4 096 wide, 32 heads over 8 of 128; the inner width and
     the vocabulary no powers of two) in true float32: whole prompts of 1 to 150 tokens against the float64 plain
