@@ -233,7 +233,8 @@ class CacheManager:
     # ---- growth ---------------------------------------------------------------------------
     def reserve(self, growth: Mapping[int, int]) -> None:
         """Makes room for `growth[slot]` more tokens in every slot named, or raises CacheFull
-        before anything has changed."""
+        before anything has changed.  What a group uploads for it (new block-table entries) is queued on the
+        current stream without a wait: call this with the stream current on which the step's kernels run."""
         for g in self.groups:
             missing = sum(g.blocks_missing(slot, self.lengths[slot] + n) for slot, n in growth.items())
             if missing > g.free_blocks():
