@@ -227,6 +227,28 @@ def test_a_freed_block_goes_to_a_survivor_while_a_step_is_queued_and_a_batch_fol
     helpers.stopping_scenarios(eng)
 
 
+def test_many_requests_of_random_lengths_through_captured_steps_equal_direct_steps(tmp_path_factory):
+    """Dozens of requests of random lengths with stop ids that end sequences at random steps, batches one after
+    another on reused slots, in a pool that just holds a batch: captured steps queued one ahead of the host (their
+    block-table entries and step arrays go up without waiting for the device) give the tokens of direct steps."""
+    import random
+
+    rng = random.Random(11)
+    folder = write_folder(tmp_path_factory.mktemp("many"), TINY_C, seed=3, std=0.05)
+    vocab = TINY_C["vocab_size"]
+    for trial in range(4):
+        n_req, new = rng.randrange(8, 30), rng.randrange(5, 70)
+        prompts = [random_tokens(rng.randrange(1, 180), vocab, 1000 * trial + i) for i in range(n_req)]
+        need = 64 * ((max(len(p) for p in prompts) + new + 63) // 64)
+        eng = lq.load_engine(folder, dtype="float32", max_tokens=need * rng.randrange(1, 4), max_sequence_tokens=4096)
+        stops = [rng.randrange(vocab) for _ in range(rng.randrange(0, 10))]
+        max_batch = rng.randrange(1, 12)
+        direct = lq.generate(eng, prompts, new, stop_ids=stops, max_batch=max_batch, use_graphs=False)
+        captured = lq.generate(eng, prompts, new, stop_ids=stops, max_batch=max_batch, use_graphs=True)
+        assert captured.tokens == direct.tokens and captured.finish == direct.finish, trial
+        assert eng.cache.free_blocks() == eng.cache.n_blocks and eng.cache.slots.taken_count == 0
+
+
 @pytest.mark.parametrize("n_prompts,max_batch", [(6, 3), (2, 1)])
 def test_batches_of_one_size_one_after_another_through_captured_graphs(tmp_path_factory, n_prompts, max_batch):
     """The second batch finds a captured graph of its own size, on the same slots, whose arrays still hold
