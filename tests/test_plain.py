@@ -167,7 +167,9 @@ def test_llama3_blend_at_hand_worked_points():
     high 4 and factor 8, original / wavelength = 2.5 gives s = (2.5 - 1) / (4 - 1) = 0.5 and
     f' = 0.5 f / 8 + 0.5 f = 0.5625 f; 1.75 gives s = 0.25 and f' = 0.75 f / 8 + 0.25 f = 0.34375 f.
     (A blend linear in the wavelength would give 0.825 f and 0.5 f.)  Both the plain function and the
-    engine's table are held to these."""
+    engine's table are held to these.  Parity unpinned: the reference has no frequency scaling at all
+    (internal/device/kernels.metal:430-463 rotates with the base frequencies as they are), so these points hold
+    the rule as config.json's `llama3` type is read here, not a vector of the reference's."""
     from longbow_quarrel_amd.parts.rope import rotary_frequencies
 
     hd, theta = 32, 500000.0
