@@ -136,6 +136,8 @@ def main() -> int:
     def random_prompt(n: int):
         return torch.randint(0, config.vocab_size, (n,), generator=gen).tolist()
 
+    event_ms = {}  # batch size -> milliseconds a step between two events on the engine's stream (the last run of that size)
+
     def decode_run(batch: int, prompt_len: int, steps: int, warmup: int):
         """tokens a second, ms a step, mean context during the timed steps"""
         # (a point over a longer context than the configuration's: the pool holds it, the bound of one
@@ -154,12 +156,18 @@ def main() -> int:
             backend.expect_more(i + 1 < warmup)
             toks = backend.decode(slots, toks, False)
         torch.cuda.synchronize()
+        # the host's clock between two synchronisations is what is reported; a pair of events on the engine's
+        # stream around the same steps says how much of it the device itself was busy
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        first.record(engine.stream)
         t = time.perf_counter()
         for i in range(steps):
             backend.expect_more(i + 1 < steps)
             toks = backend.decode(slots, toks, False)
+        last.record(engine.stream)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
+        event_ms[batch] = first.elapsed_time(last) / steps
         ctx_mean = sum(lens) / batch + warmup + (steps + 1) / 2.0
         for s in slots:
             backend.release(s)
@@ -260,7 +268,9 @@ def main() -> int:
         value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
     step_bytes = weight_bytes_per_step(config, element) + args.batch * ctx_mean * kv_bytes_per_token(config, element)
     achieved = step_bytes / (ms_step * 1e-3) / 1e9
-    print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
+    between_events = event_ms.get(args.batch)
+    print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_step:.3f} ms/step" +
+          (f" ({between_events:.3f} ms between events on the stream)" if between_events else ""), file=sys.stderr, flush=True)
 
     if not args.no_points and not through_loop:
         prefill = prefill_point(2048)
@@ -285,7 +295,8 @@ def main() -> int:
             f"prompts of {args.prompt_len} to {args.prompt_len_max} tokens)" if args.prompt_len_max > args.prompt_len
             else f"{args.prompt_len}-token prompts)"),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_step, 4), "ms_per_step_events": round(between_events, 4) if between_events else None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if element == 2 else "fp32", "data": "synthetic: random weights N(0, 0.02) from a seed, uniform random token ids",
         "config": {
             "model": f"llama3-{args.shape}-shape", "layers": config.num_hidden_layers, "layers_full": full_layers,
