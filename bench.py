@@ -9,9 +9,10 @@ greedy sampling on the device and state upkeep, replayed as a HIP graph, tokens 
 back by the host every step as generation does).  `value` is decoded tokens a
 second.  The same line carries a 2,048-token prefill, the decode step's HBM
 roofline, and as `points` decode at batch 1 and 64, prefills of 512 and 8,192 tokens
-(tokens a second) and decode at batch 8 from prompts of 8,192 and 32,768 tokens (the
+(tokens a second), decode at batch 8 from prompts of 8,192 and 32,768 tokens (the
 pool of the 64 x 8,192-token cache holds them; only the bound of one sequence is raised
-for these).  One JSON line on stdout.
+for these), and the 1B shape's workload of `--shape 1b` with an engine of its own.  One
+JSON line on stdout.
 
 `--dtype float32` runs the true 32-bit path (float32 weights, cache and activations; peaks:
 157.3 TFLOP/s, the same 8 TB/s); with the 8B shape that is for a few layers (`--layers 4`).
@@ -244,26 +245,29 @@ def main() -> int:
 
     prefill = None
     points = {}
-    if through_loop:
-        # 16 prompts of unequal lengths, then decoding, as one call of the generation loop; the untimed
-        # call before it leaves the captured steps behind for the timed one
-        lens = torch.randint(args.prompt_len, args.prompt_len_max + 1, (args.batch,), generator=gen).tolist()
-        prompts = [random_prompt(n) for n in lens]
-        backend = EngineBackend(engine, lq.SamplingParams(temperature=0.0), use_graphs=True)
-        loop = GenerationLoop(backend, max_batch=args.batch)
-        loop.run(prompts, args.warmup + 1, stop_ids=[])
+    def loop_run(eng, conf, batch, lo, hi, steps, warmup):
+        """`batch` prompts of lengths uniform in [lo, hi], then `steps` decoding steps, as one call of the
+        generation loop; the untimed call before it leaves the captured steps behind for the timed one.
+        -> tokens a second, ms a step, mean context, the prompts' figures"""
+        lens = torch.randint(lo, hi + 1, (batch,), generator=gen).tolist()
+        prompts = [torch.randint(0, conf.vocab_size, (n,), generator=gen).tolist() for n in lens]
+        backend = EngineBackend(eng, lq.SamplingParams(temperature=0.0), use_graphs=True)
+        loop = GenerationLoop(backend, max_batch=batch)
+        loop.run(prompts, warmup + 1, stop_ids=[])
         torch.cuda.synchronize()
-        res = loop.run(prompts, args.steps + 1, stop_ids=[])  # the first token comes from the prompts' step
+        res = loop.run(prompts, steps + 1, stop_ids=[])  # the first token comes from the prompts' step
         backend.close()
-        assert res.decode_steps == args.steps and res.batches == 1
-        ms_step = res.decode_seconds / res.decode_steps * 1e3
-        value = args.batch * res.decode_steps / res.decode_seconds
-        ctx_mean = sum(lens) / args.batch + (args.steps + 1) / 2.0
-        n_prompt = res.prefill_tokens
-        flops = sum(prefill_flops(config, n) for n in lens)
-        prefill = {"value": round(n_prompt / res.prefill_seconds, 1), "tokens": n_prompt,
-                   "ms": round(res.prefill_seconds * 1e3, 3),
-                   "frac": round(flops / res.prefill_seconds / (peak_tflops * 1e12), 4)}
+        assert res.decode_steps == steps and res.batches == 1
+        flops = sum(prefill_flops(conf, n) for n in lens)
+        prompts_line = {"value": round(res.prefill_tokens / res.prefill_seconds, 1), "tokens": res.prefill_tokens,
+                        "ms": round(res.prefill_seconds * 1e3, 3),
+                        "frac": round(flops / res.prefill_seconds / (peak_tflops * 1e12), 4)}
+        return (batch * res.decode_steps / res.decode_seconds, res.decode_seconds / res.decode_steps * 1e3,
+                sum(lens) / batch + (steps + 1) / 2.0, prompts_line)
+
+    if through_loop:
+        value, ms_step, ctx_mean, prefill = loop_run(engine, config, args.batch, args.prompt_len, args.prompt_len_max,
+                                                     args.steps, args.warmup)
     else:
         value, ms_step, ctx_mean = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
     step_bytes = weight_bytes_per_step(config, element) + args.batch * ctx_mean * kv_bytes_per_token(config, element)
@@ -288,6 +292,16 @@ def main() -> int:
                 if args.batch * (ctx + 64) <= max_batch * slot_len:
                     v, _, _ = decode_run(args.batch, ctx, max(8, args.steps // 4), max(2, args.warmup // 4))
                     points[f"decode_b{args.batch}_ctx{ctx}"] = round(v, 1)
+            # the 1B shape's workload (16 prompts of 64 to 4,096 tokens through the generation loop), with an
+            # engine of its own beside this one: what `--shape 1b` runs, with fewer steps
+            small = lq.LlamaConfig.from_dict(dict(CONFIG_1B))
+            engine_1b = lq.random_engine(small, seed=0, dtype="bfloat16", max_tokens=16 * 8192, max_slots=16)
+            v, ms, ctx, line_1b = loop_run(engine_1b, small, 16, 64, 4096, max(16, args.steps // 2), max(4, args.warmup // 2))
+            bytes_1b = weight_bytes_per_step(small) + 16 * ctx * kv_bytes_per_token(small)
+            points["decode_1b_b16"] = round(v, 1)
+            points["decode_1b_b16_hbm_frac"] = round(bytes_1b / (ms * 1e-3) / 1e9 / HBM_GBPS, 4)
+            points["prefill_1b"] = line_1b["value"]
+            del engine_1b
         print(f"[bench] points: {points}", file=sys.stderr, flush=True)
 
     line = {
