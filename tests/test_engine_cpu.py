@@ -151,8 +151,14 @@ def test_toy_parts_register_build_and_step_without_touching_the_framework(tmp_pa
         sa, sb = eng.new_sequence(), eng.new_sequence()
         out = eng.step([StepEntry(sa, a[:17], range(17)), StepEntry(sb, b[:8], range(8))])
         assert rel_err(out[:17], wa[:17]) < TOL and rel_err(out[17:], wb[:8]) < TOL
+        # what a captured step is keyed by is the mixers' answer: the toy's own rule (steps of 500 tokens, uneven
+        # beyond three to one) beside attention's default
+        assert eng.length_bound(5) == 500 and eng.length_bound(501) == 1000
+        assert eng.lengths_uneven([40, 10]) and not eng.lengths_uneven([30, 10])
+        del toy_parts.DecayMixer.seen[:]
         out = eng.step([StepEntry(sa, a[17:18], [0]), StepEntry(sb, b[8:], [0])])
         assert rel_err(out[0], wa[17]) < TOL and rel_err(out[1], wb[8]) < TOL
+        assert toy_parts.DecayMixer.seen == [(18, False)]  # a direct step: the longest length itself, 18 to 9
         eng.release(sb)
         out = eng.step([StepEntry(sa, a[18:], range(22))])
         assert rel_err(out, wa[18:]) < TOL

@@ -36,7 +36,19 @@ class DecayMixer(Mixer):
     def cache_need(self) -> StateNeed:
         return StateNeed((self.width,), torch.float32)
 
+    # a rule of its own for what a captured decoding step is keyed by: bounds in steps of 500 tokens, and
+    # "uneven" where one sequence holds more than three times another's tokens
+    def length_bound(self, kernels, longest: int) -> int:
+        return -(-longest // 500) * 500
+
+    def lengths_uneven(self, kernels, lengths) -> bool:
+        return max(lengths) > 3 * min(lengths)
+
+    seen: List = []  # (max_len, uneven) of the decoding steps that reached forward
+
     def forward(self, h: torch.Tensor, ctx: StepContext, cache: Optional[LayerCache]) -> torch.Tensor:
+        if ctx.rows == len(ctx.host_slots):
+            DecayMixer.seen.append((ctx.max_len, ctx.uneven))
         states = torch.empty((ctx.rows, self.width), dtype=torch.float32, device=h.device)
         row = 0
         for slot, n in zip(ctx.host_slots, ctx.host_new):
