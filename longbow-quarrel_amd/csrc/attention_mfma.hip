@@ -91,6 +91,14 @@ __device__ inline float rows_sum(float x) {
 // probability that small is worth)
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The running maximum that the probabilities are taken against follows the scores' maximum lazily: it moves
+// (and what has been summed is rescaled) only when some row of the wave meets a score more than this far
+// above it, in the log2 domain.  Probabilities then reach 2^8 at most, which float32 sums and bfloat16
+// operands (eight bits of exponent) hold as well as values below 1; the quotient at the end is the same.
+// After a row's first keys the branch is taken rarely; with a slack of zero it ran whenever any row's maximum
+// moved at all, and its multiplications of every accumulator cost 5 to 8 % of a long prompt's time.
+constexpr float RESCALE_SLACK = 8.0f;
+
 // Which key of a 32-key chunk row r of score tile j stands for: the rows are dealt out so that the
 // eight probabilities a lane ends up with (rows (lane/16)*4 + e of both tiles) belong to eight
 // consecutive keys, (lane/16)*8 .. +7: the second product then takes its V^T operand as one
@@ -120,18 +128,22 @@ __device__ inline float softmax_chunk(const f32x4 (&s)[2], float c, bool masked,
       }
   }
   float cmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-  cmax = rows_max(cmax);
-  const float m_new = fmaxf(m, cmax * c);  // c > 0: scaling commutes with the maximum
-  const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a column with no key yet
-  const float alpha = fast_exp2(m - m_safe);
+  cmax = rows_max(cmax) * c;  // c > 0: scaling commutes with the maximum
+  float alpha = 1.0f;
+  if (__any(cmax > m + RESCALE_SLACK)) {  // (false for -inf against -inf, true for anything against -inf)
+    const float m_new = fmaxf(m, cmax);
+    alpha = fast_exp2(m - ((m_new == -INFINITY) ? 0.f : m_new));
+    l *= alpha;
+    m = m_new;
+  }
+  const float m_safe = (m == -INFINITY) ? 0.f : m;  // a column with no key yet
   float psum = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     sv[i] = fast_exp2(fmaf(sv[i], c, -m_safe));  // -inf stays -inf, 2^-inf = 0
     psum += sv[i];
   }
-  l = l * alpha + psum;
-  m = m_new;
+  l += psum;
   pw[0] = pack_bf16(sv[0], sv[1]);
   pw[1] = pack_bf16(sv[2], sv[3]);
   pw[2] = pack_bf16(sv[4], sv[5]);
@@ -683,28 +695,30 @@ __global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int
         auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(cmax), __float_as_uint(cmax), false, false);
         cmax = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
       }
-      const float m_new = fmaxf(m, cmax * a.scale_log2);  // the scale is positive: it commutes with the maximum
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row with no key yet
-      const float alpha = fast_exp2(m - m_safe);
+      cmax *= a.scale_log2;  // the scale is positive: it commutes with the maximum
+      if (__any(cmax > m + RESCALE_SLACK)) {  // some row's maximum moved far: rescale what has been summed
+        const float m_new = fmaxf(m, cmax);
+        const float alpha = fast_exp2(m - ((m_new == -INFINITY) ? 0.f : m_new));
+        l *= alpha;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+      }
+      const float m_safe = (m == -INFINITY) ? 0.f : m;  // a row with no key yet
       float psum = 0.f;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         sc[e] = fast_exp2(fmaf(sc[e], a.scale_log2, -m_safe));  // -inf stays -inf, 2^-inf = 0
         psum += sc[e];
       }
-      l = l * alpha + psum;
-      m = m_new;
+      l += psum;
       u32x4 pw[2];
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int j = 0; j < 4; ++j) pw[s2][j] = pack_bf16(sc[8 * s2 + 2 * j], sc[8 * s2 + 2 * j + 1]);
-      if (!__all(alpha == 1.0f)) {  // the maximum moved for some row: rescale what has been summed
-#pragma unroll
-        for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
-      }
       const unsigned char* vr = cur + L::K_BYTES + c32 * L::V_STRIDE + half * 64 + hf * 16;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)

@@ -283,9 +283,10 @@ def test_linear_row_does_not_depend_on_the_batch(kn):
 BS = 64
 
 
-def paged_cache(lengths, kv_heads, head_dim, dtype, seed):
+def paged_cache(lengths, kv_heads, head_dim, dtype, seed, ramp=None):
     """Random keys/values for sequences of the given lengths in a paged cache whose blocks are
-    handed out in a shuffled order; returns dense copies too."""
+    handed out in a shuffled order; returns dense copies too.  With `ramp` the keys' first component is
+    ramp(t) at position t."""
     g = torch.Generator().manual_seed(seed)
     need = [(n + BS - 1) // BS for n in lengths]
     n_blocks = sum(need) + 3
@@ -296,7 +297,10 @@ def paged_cache(lengths, kv_heads, head_dim, dtype, seed):
     vc = torch.zeros((n_blocks, kv_heads, head_dim, BS), dtype=dtype)
     dense = []
     for b, n in enumerate(lengths):
-        k = torch.randn((n, kv_heads, head_dim), generator=g).to(dtype)
+        k = torch.randn((n, kv_heads, head_dim), generator=g)
+        if ramp is not None:
+            k[:, :, 0] = torch.tensor([ramp(t) for t in range(n)])[:, None]
+        k = k.to(dtype)
         v = torch.randn((n, kv_heads, head_dim), generator=g).to(dtype)
         dense.append((k, v))
         for j in range(need[b]):
@@ -309,15 +313,20 @@ def paged_cache(lengths, kv_heads, head_dim, dtype, seed):
 
 
 def run_attention(kn, q_rows, lengths, new, heads, kv_heads, head_dim, dtype, seed, window=0, decode=False,
-                  force_generic=False, standout=None, max_len=None, uneven=False, check=None, q_by_position=False):
+                  force_generic=False, standout=None, max_len=None, uneven=False, check=None, q_by_position=False,
+                  ramp=None):
     """q rows for the last `new[b]` positions of each sequence; returns (got, want).  With `check` (rows of
     the step, counted through all sequences) only these rows are worked out by the plain implementation
     and returned: for steps of thousands of rows.  With `q_by_position` the query of a position of a sequence is
-    the same whatever rows the step brings (for comparisons between steps)."""
-    kc, vc, table, slots, dense = paged_cache(lengths, kv_heads, head_dim, dtype, seed)
+    the same whatever rows the step brings (for comparisons between steps).  With `ramp` the scores of a
+    row grow with the key's position by ramp(t) (natural-log units) on top of the random part."""
+    kc, vc, table, slots, dense = paged_cache(lengths, kv_heads, head_dim, dtype, seed, ramp)
     g = torch.Generator().manual_seed(seed + 1)
     rows = sum(new)
-    q = torch.randn((rows, heads * head_dim), generator=g).to(dtype)
+    q = torch.randn((rows, heads * head_dim), generator=g)
+    if ramp is not None:
+        q.view(rows, heads, head_dim)[:, :, 0] = math.sqrt(head_dim)  # times the scale: 1
+    q = q.to(dtype)
     if q_by_position:
         per_seq = [torch.randn((n, heads * head_dim), generator=torch.Generator().manual_seed(seed + 7 + b)).to(dtype)
                    for b, n in enumerate(lengths)]
@@ -373,6 +382,20 @@ def test_attention_prompts(kn, dtype, generic, heads, kv_heads, head_dim):
     got, want = run_attention(kn, None, [5, 70, 131, 1], [5, 70, 40, 1], heads, kv_heads, head_dim, dtype, 21,
                               force_generic=generic)
     assert rel_err(got, want) < (2e-6 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(8, 2, 64), (8, 2, 128), (4, 4, 128), (2, 1, 96)])
+@pytest.mark.parametrize("shape", ["slow", "steps", "down"])
+def test_attention_when_the_largest_score_keeps_moving(kn, heads, kv_heads, head_dim, shape):
+    """The running maximum of the prompt kernels follows the scores lazily (it moves when a score stands far
+    enough above it).  Scores that creep up by less than that a chunk, that jump by more every few hundred
+    keys, and that fall from a large first key all give the plain implementation's result."""
+    ramp = {"slow": lambda t: 0.05 * t,                       # 2.3 in the log2 domain every 32 keys
+            "steps": lambda t: 9.0 * (t // 200),              # 13 in the log2 domain every 200 keys
+            "down": lambda t: 40.0 - 0.03 * t}[shape]
+    got, want = run_attention(kn, None, [700, 333, 40], [700, 300, 40], heads, kv_heads, head_dim, torch.bfloat16, 57,
+                              ramp=ramp)
+    assert rel_err(got, want) < 8e-3
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,lengths,new,window", [
