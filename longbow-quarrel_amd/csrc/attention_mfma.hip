@@ -397,10 +397,10 @@ __global__ __launch_bounds__(HW * RT * 64, (HD <= 128 && HW * RT > 1 ? 2 : 1)) v
     const int first_pos = p0 + min((tile0 + qt) * 16, nrows - 1);
     w.last_key[qt] = (wave_active && rows_here > 0) ? p0 + (tile0 + qt) * 16 + rows_here - 1 : -1;
     w.first_key[qt] = (a.window > 0 && first_pos >= a.window) ? first_pos - a.window + 1 : 0;
-    // a full tile of 16 rows: keys up to its first row's position and from its last row's window
-    // start on are visible to all of its columns
+    // keys up to the tile's first row's position and from its last row's window start on are visible to
+    // all of its columns (those past a partial tile's rows run as copies of its last row, never stored)
     const int last_pos = p0 + (tile0 + qt) * 16 + rows_here - 1;
-    w.free_to[qt] = (wave_active && rows_here == 16) ? first_pos : -1;
+    w.free_to[qt] = (wave_active && rows_here > 0) ? first_pos : -1;
     w.free_from[qt] = (a.window > 0 && last_pos >= a.window) ? last_pos - a.window + 1 : 0;
     const bf16_t* qr = a.q + (long long)row * a.ldq + h * HD + g * 8;
 #pragma unroll
@@ -599,7 +599,8 @@ __global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int
   const int last_key = wave_active ? p0 + nrows - 1 : -1;                       // wave-uniform
   const int first_key = (a.window > 0 && p0 >= a.window) ? p0 - a.window + 1 : 0;
   // keys up to the first row's position and from the last row's window start on are visible to all 32 rows
-  const int free_to = (wave_active && nrows == ROWS) ? p0 : -1;
+  // (the columns past a partial tile run as copies of its last row and are never stored: they see these keys too)
+  const int free_to = wave_active ? p0 : -1;
   const int free_from = (a.window > 0 && p0 + nrows - 1 >= a.window) ? p0 + nrows - 1 - a.window + 1 : 0;
   bf16x8 q[HD / 16];
   {
@@ -677,9 +678,22 @@ __global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int
 #pragma unroll
       for (int e = 0; e < 16; ++e) sc[e] = 0.f;
       const unsigned char* kr = cur + (half * 32 + c32) * L::K_STRIDE + hf * 16;
+      const unsigned char* vr = cur + L::K_BYTES + c32 * L::V_STRIDE + half * 64 + hf * 16;
+      // All of the half's K fragments are asked for before the first product, and its V^T fragments as soon
+      // as the products have been issued, so that they arrive during the products and the softmax: a wave
+      // that asks for each fragment just before its product waits out the LDS latency sixteen times a half.
+      u32x4 kf[HD / 16], vf[2][HD / 32];
+#pragma unroll
+      for (int kk = 0; kk < HD / 16; ++kk) kf[kk] = *(const u32x4*)(kr + kk * 32);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int kk = 0; kk < HD / 16; ++kk)
-        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(*(const u32x4*)(kr + kk * 32)), q[kk], sc, 0, 0, 0);
+        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kk]), q[kk], sc, 0, 0, 0);
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) vf[s2][dt] = *(const u32x4*)(vr + dt * 32 * L::V_STRIDE + s2 * 32);
+      __builtin_amdgcn_sched_barrier(0);
       const bool masked = !(t0 + 31 <= free_to && t0 >= free_from);
       if (masked) {
 #pragma unroll
@@ -719,13 +733,11 @@ __global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int j = 0; j < 4; ++j) pw[s2][j] = pack_bf16(sc[8 * s2 + 2 * j], sc[8 * s2 + 2 * j + 1]);
-      const unsigned char* vr = cur + L::K_BYTES + c32 * L::V_STRIDE + half * 64 + hf * 16;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt)
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(*(const u32x4*)(vr + dt * 32 * L::V_STRIDE + s2 * 32)),
-                                                          as_bf16x8(pw[s2]), o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(vf[s2][dt]), as_bf16x8(pw[s2]), o[dt], 0, 0, 0);
     }
     // Nobody reads nxt: its last readers passed the barrier below one round ago.
     if (more) stash(lb + 1, nxt);
@@ -1153,16 +1165,16 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
     if constexpr (HD % 32 == 0 && HD <= 128) {
       // The 32 x 32 score tile (its accumulators fit up to this head size) reads half as much from LDS for a
       // product, with half as many waves on a compute unit to hide one wave's softmax behind another's
-      // products.  As measured (32 heads over 8, one sequence): at head size 64 it wins at every length
-      // (46 against 68 us at 2 048 tokens, 353 against 429 at 8 192), at 96 and 128 from about 3 000 tokens a
-      // sequence on (644 against 682 us at 8 192, 76 against 68 at 2 048); with fewer than four heads a
-      // kv head it wins throughout.
-      const bool wide = HD <= 64 || G < 4 || rows >= 3072 * a.batch;
-      if (wide && G >= 4) return launch_rows32<HD, 4>(a, rows, lq_ceil_div(G, 4), stream);
-      if (wide && G >= 2) return launch_rows32<HD, 2>(a, rows, lq_ceil_div(G, 2), stream);
-      // (one wave a block would have to stage a whole cache block through its own registers)
-      if constexpr (HD <= 64)
-        if (wide && G == 1) return launch_rows32<HD, 1>(a, rows, 1, stream);
+      // products.  As measured (32 heads over 8): at head size 64 it wins at every length (46 against 68 us at
+      // 2 048 tokens, 353 against 429 at 8 192); at head size 128 it wins or ties at every length too (one
+      // sequence of 256 tokens 16.7 against 16.6 us, of 1 000 tokens 33.8 against 34.2, of 2 048 tokens 65.9
+      // against 67.7, of 8 192 tokens 612 against 682; sixteen sequences of 512 tokens 79 against 84, eight of 300
+      // tokens 29.0 against 28.5) since its fragments are asked for early and partial tiles take the unmasked
+      // path below the diagonal.  With one head a kv head a workgroup would be one wave that stages a whole
+      // cache block through its own registers: then the narrow tiles stay for head sizes above 64.
+      if (G >= 4) return launch_rows32<HD, 4>(a, rows, lq_ceil_div(G, 4), stream);
+      if (G >= 2) return launch_rows32<HD, 2>(a, rows, lq_ceil_div(G, 2), stream);
+      if constexpr (HD <= 64) return launch_rows32<HD, 1>(a, rows, 1, stream);
     }
     if (G >= 4) return launch_rows<HD, QT2, 4, 2>(a, rows, lq_ceil_div(G, 4), stream);
     if (G >= 2) return launch_rows<HD, QT, 2, 1>(a, rows, lq_ceil_div(G, 2), stream);

@@ -396,19 +396,29 @@ def test_attention_when_the_largest_score_keeps_moving(kn, heads, kv_heads, head
     got, want = run_attention(kn, None, [700, 333, 40], [700, 300, 40], heads, kv_heads, head_dim, torch.bfloat16, 57,
                               ramp=ramp)
     assert rel_err(got, want) < 8e-3
+    if (heads, head_dim) == (8, 128):  # a long sequence too
+        got, want = run_attention(kn, None, [2650], [2650], heads, kv_heads, head_dim, torch.bfloat16, 58, ramp=ramp,
+                                  check=[0, 40, 700, 1999, 2000, 2001, 2649])
+        assert rel_err(got, want) < 8e-3
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,lengths,new,window", [
     (8, 2, 64, [5, 70, 131, 1, 300], [5, 70, 40, 1, 300], 0),   # four heads a kv head, head size 64: 32 x 32 tiles
     (8, 2, 64, [200, 333], [200, 100], 90),                      # and with a window
-    (16, 2, 128, [3100], [3100], 0),                             # head size 128: 32 x 32 tiles from 3 072 rows a sequence
+    (16, 2, 128, [3100], [3100], 0),                             # head size 128: 32 x 32 tiles as well
     (8, 2, 128, [3200], [3200], 1000),
-    (8, 2, 96, [100, 3200 * 2 - 100], [100, 3200 * 2 - 100], 0), # two sequences, 3 200 rows on average
-    (8, 2, 128, [700, 64, 257], [700, 64, 200], 0),              # short sequences of head size 128: 16 x 16 tiles
+    (8, 2, 96, [100, 3200 * 2 - 100], [100, 3200 * 2 - 100], 0), # two sequences, one short
+    (8, 2, 128, [300] * 9, [300] * 9, 0),                        # many short sequences with partial last tiles
+    (8, 2, 128, [700, 64, 257], [700, 64, 200], 0),
+    (8, 2, 192, [700, 64, 257, 1], [700, 64, 200, 1], 0),        # head sizes above 128: 16 x 16 tiles, four heads a kv head
+    (8, 2, 192, [333, 200], [100, 200], 90),                     # ... with a window, partial tiles
+    (4, 1, 256, [300, 45], [300, 45], 0),
+    (3, 3, 128, [700, 77], [700, 77], 0),                        # one head a kv head at head size 128: 16 x 16 tiles
+    (6, 3, 96, [700, 77], [650, 77], 100),                       # two heads a kv head
 ])
 def test_attention_prompts_on_both_tile_shapes(kn, heads, kv_heads, head_dim, lengths, new, window):
     """Prompt attention has a kernel with 32 x 32 score tiles and one with 16 x 16: which one runs depends on
-    the head size, the heads a kv head and the rows a sequence.  Both against the plain implementation."""
+    the head size, the heads a kv head and the rows of the step.  Both against the plain implementation."""
     got, want = run_attention(kn, None, lengths, new, heads, kv_heads, head_dim, torch.bfloat16, 77, window=window)
     assert rel_err(got, want) < 8e-3
 
