@@ -556,11 +556,17 @@ int launch_rows(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
 //   the keys of every 16 in the order [0-3][8-11][4-7][12-15], which makes those eight one 16-byte run.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-template <int HD, int HW>
-__global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int heads_per_block_group, int tiles,
-                                                                 int units) {
+// With KS = 2 a head's 32 rows are shared by two waves that take the first and the second 32 keys of every
+// cache block and add their results up through LDS at the end: a tile's time is set by its last row tile's
+// walk through all the keys before it, and on a short prompt, where the chip holds every tile at once, that
+// walk is the launch's time.
+template <int HD, int HW, int KS>
+__global__ __launch_bounds__(HW * KS * 64, KS == 2 ? 1 : 2) void attn_rows32_kernel(AttnArgs a, int heads_per_block_group,
+                                                                                   int tiles, int units) {
   using L = RowsLds<HD>;
-  constexpr int ROWS = 32, THREADS = HW * 64;
+  constexpr int ROWS = 32, THREADS = HW * KS * 64;
+  constexpr int MERGE_FLOATS = HD / 32 * 16 * 64 + 2 * 64;  // a wave's accumulators, maxima and normaliser shares
+  static_assert(KS == 1 || (KS == 2 && HW * MERGE_FLOATS * 4 <= 2 * L::STAGE), "the second waves' results fit the stages");
   constexpr int PER_THREAD = (L::PIECES + THREADS - 1) / THREADS;  // pieces of K, and of V, per thread
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -583,9 +589,10 @@ __global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int
   }
   if (r0 < 0) return;  // the whole block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c32 = lane & 31, hf = lane >> 5;
+  const int head_slot = wave % HW, ks = wave / HW;  // (ks: which 32 keys of a cache block, with KS = 2)
   const int G = a.nh / a.nkv;
   const int kvh = head_group / heads_per_block_group;
-  const int hq = (head_group % heads_per_block_group) * HW + wave;
+  const int hq = (head_group % heads_per_block_group) * HW + head_slot;
   const bool wave_active = hq < G;  // an idle wave still copies and meets the barriers
   const int h = kvh * G + min(hq, G - 1);
   const int* table = a.block_table + (long long)a.seq_slot[b] * a.bt_stride;
@@ -670,7 +677,8 @@ __global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int
     const bool more = lb < blk_last;
     if (more) fetch(lb + 1);  // on their way during this block's products
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
+    for (int hh = 0; hh < 2 / KS; ++hh) {
+      const int half = KS == 2 ? ks : hh;
       const int t0 = lb * BS + half * 32;
       if (t0 > t_end) break;
       if (t0 > last_key || t0 + 31 < first_key) continue;  // nothing of this chunk is visible to this wave
@@ -743,6 +751,29 @@ __global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int
     if (more) stash(lb + 1, nxt);
     __syncthreads();
   }
+  if constexpr (KS == 2) {
+    // the second waves' sums go to the first through LDS (everyone is past the last stage's reads)
+    float* mine = (float*)smem + head_slot * MERGE_FLOATS;
+    if (ks == 1) {
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mine[(dt * 16 + e) * 64 + lane] = o[dt][e];
+      mine[HD / 32 * 16 * 64 + lane] = m;
+      mine[HD / 32 * 16 * 64 + 64 + lane] = l;
+    }
+    __syncthreads();
+    if (ks == 1) return;
+    const float m1 = mine[HD / 32 * 16 * 64 + lane], l1 = mine[HD / 32 * 16 * 64 + 64 + lane];
+    const float m_all = fmaxf(m, m1);
+    const float m_safe = (m_all == -INFINITY) ? 0.f : m_all;
+    const float f0 = fast_exp2(m - m_safe), f1 = fast_exp2(m1 - m_safe);  // 2^-inf = 0: a wave that saw no key
+    l = l * f0 + l1 * f1;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[dt][e] = o[dt][e] * f0 + mine[(dt * 16 + e) * 64 + lane] * f1;
+  }
   {
     auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l), __float_as_uint(l), false, false);
     l = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
@@ -761,11 +792,11 @@ __global__ __launch_bounds__(HW * 64, 2) void attn_rows32_kernel(AttnArgs a, int
     }
 }
 
-template <int HD, int HW>
+template <int HD, int HW, int KS>
 int launch_rows32(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
   using L = RowsLds<HD>;
   const size_t smem = 2 * (size_t)L::STAGE;
-  auto kernel = attn_rows32_kernel<HD, HW>;
+  auto kernel = attn_rows32_kernel<HD, HW, KS>;
   static bool configured = false;
   if (!configured && smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -776,7 +807,7 @@ int launch_rows32(const AttnArgs& a, int rows, int groups, hipStream_t stream) {
     configured = true;
   }
   const int tiles = lq_ceil_div(rows, 32) + a.batch;  // an upper bound: a sequence's last tile may be partial
-  kernel<<<dim3(tiles * a.nkv * groups), HW * 64, smem, stream>>>(a, groups, tiles, lq_compute_units());
+  kernel<<<dim3(tiles * a.nkv * groups), HW * KS * 64, smem, stream>>>(a, groups, tiles, lq_compute_units());
   LQ_CHECK_LAUNCH("attention(mfma rows, 32 x 32)");
   return 0;
 }
@@ -1172,9 +1203,21 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
       // tokens 29.0 against 28.5) since its fragments are asked for early and partial tiles take the unmasked
       // path below the diagonal.  With one head a kv head a workgroup would be one wave that stages a whole
       // cache block through its own registers: then the narrow tiles stay for head sizes above 64.
-      if (G >= 4) return launch_rows32<HD, 4>(a, rows, lq_ceil_div(G, 4), stream);
-      if (G >= 2) return launch_rows32<HD, 2>(a, rows, lq_ceil_div(G, 2), stream);
-      if constexpr (HD <= 64) return launch_rows32<HD, 1>(a, rows, 1, stream);
+      // Two waves a head (each half of every cache block's keys) where the workgroups would not even be one a
+      // compute unit: the chip then holds twice the waves and a tile's walk through its keys takes half as
+      // long (one sequence of 1 000 tokens 32.6 -> 28.5 us, of 700 tokens 24.8 -> 22.2).  With more workgroups
+      // than that they would run one after the other, eight waves each, where two of four waves run side by
+      // side (2 048 tokens 64.8 -> 72.8 us, 8 192 tokens 597 -> 648).
+      const int hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
+      const bool two = (long long)lq_ceil_div(rows, 32) * a.nkv * lq_ceil_div(G, hw) <= lq_compute_units();
+      if (G >= 4)
+        return two ? launch_rows32<HD, 4, 2>(a, rows, lq_ceil_div(G, 4), stream)
+                   : launch_rows32<HD, 4, 1>(a, rows, lq_ceil_div(G, 4), stream);
+      if (G >= 2)
+        return two ? launch_rows32<HD, 2, 2>(a, rows, lq_ceil_div(G, 2), stream)
+                   : launch_rows32<HD, 2, 1>(a, rows, lq_ceil_div(G, 2), stream);
+      if constexpr (HD <= 64)
+        return two ? launch_rows32<HD, 1, 2>(a, rows, 1, stream) : launch_rows32<HD, 1, 1>(a, rows, 1, stream);
     }
     if (G >= 4) return launch_rows<HD, QT2, 4, 2>(a, rows, lq_ceil_div(G, 4), stream);
     if (G >= 2) return launch_rows<HD, QT, 2, 1>(a, rows, lq_ceil_div(G, 2), stream);

@@ -410,6 +410,8 @@ def test_attention_when_the_largest_score_keeps_moving(kn, heads, kv_heads, head
     (8, 2, 96, [100, 3200 * 2 - 100], [100, 3200 * 2 - 100], 0), # two sequences, one short
     (8, 2, 128, [300] * 9, [300] * 9, 0),                        # many short sequences with partial last tiles
     (8, 2, 128, [700, 64, 257], [700, 64, 200], 0),
+    (32, 8, 128, [1100, 333], [1100, 300], 0),                   # more workgroups than compute units: a wave a head
+    (16, 8, 128, [1500, 77], [1500, 77], 500),                   # ... two heads a kv head, a window
     (8, 2, 192, [700, 64, 257, 1], [700, 64, 200, 1], 0),        # head sizes above 128: 16 x 16 tiles, four heads a kv head
     (8, 2, 192, [333, 200], [100, 200], 90),                     # ... with a window, partial tiles
     (4, 1, 256, [300, 45], [300, 45], 0),
@@ -417,8 +419,9 @@ def test_attention_when_the_largest_score_keeps_moving(kn, heads, kv_heads, head
     (6, 3, 96, [700, 77], [650, 77], 100),                       # two heads a kv head
 ])
 def test_attention_prompts_on_both_tile_shapes(kn, heads, kv_heads, head_dim, lengths, new, window):
-    """Prompt attention has a kernel with 32 x 32 score tiles and one with 16 x 16: which one runs depends on
-    the head size, the heads a kv head and the rows of the step.  Both against the plain implementation."""
+    """Prompt attention has a kernel with 32 x 32 score tiles (a wave a head, or two that share a cache block's
+    keys where the step has few rows) and one with 16 x 16: which one runs depends on the head size, the heads
+    a kv head and the rows of the step.  All against the plain implementation."""
     got, want = run_attention(kn, None, lengths, new, heads, kv_heads, head_dim, torch.bfloat16, 77, window=window)
     assert rel_err(got, want) < 8e-3
 
