@@ -249,8 +249,9 @@ def main() -> int:
         """`batch` prompts of lengths uniform in [lo, hi], then `steps` decoding steps, as one call of the
         generation loop; the untimed call before it leaves the captured steps behind for the timed one.
         -> tokens a second, ms a step, mean context, the prompts' figures"""
-        lens = torch.randint(lo, hi + 1, (batch,), generator=gen).tolist()
-        prompts = [torch.randint(0, conf.vocab_size, (n,), generator=gen).tolist() for n in lens]
+        own = torch.Generator().manual_seed(7)  # the same prompts whatever else this run has drawn before
+        lens = torch.randint(lo, hi + 1, (batch,), generator=own).tolist()
+        prompts = [torch.randint(0, conf.vocab_size, (n,), generator=own).tolist() for n in lens]
         backend = EngineBackend(eng, lq.SamplingParams(temperature=0.0), use_graphs=True)
         loop = GenerationLoop(backend, max_batch=batch)
         loop.run(prompts, warmup + 1, stop_ids=[])
