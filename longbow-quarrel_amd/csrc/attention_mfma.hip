@@ -1218,10 +1218,13 @@ int launch(const AttnArgs& a, int rows, int decode, hipStream_t stream) {
                    : launch_rows32<HD, 2, 1>(a, rows, lq_ceil_div(G, 2), stream);
       if constexpr (HD <= 64)
         return two ? launch_rows32<HD, 1, 2>(a, rows, 1, stream) : launch_rows32<HD, 1, 1>(a, rows, 1, stream);
+      else
+        return launch_rows<HD, QT, 1, 1>(a, rows, 1, stream);
+    } else {
+      if (G >= 4) return launch_rows<HD, QT2, 4, 2>(a, rows, lq_ceil_div(G, 4), stream);
+      if (G >= 2) return launch_rows<HD, QT, 2, 1>(a, rows, lq_ceil_div(G, 2), stream);
+      return launch_rows<HD, QT, 1, 1>(a, rows, 1, stream);
     }
-    if (G >= 4) return launch_rows<HD, QT2, 4, 2>(a, rows, lq_ceil_div(G, 4), stream);
-    if (G >= 2) return launch_rows<HD, QT, 2, 1>(a, rows, lq_ceil_div(G, 2), stream);
-    return launch_rows<HD, QT, 1, 1>(a, rows, 1, stream);
   }
   // Four waves a block (two where their partial outputs would not fit 48 KiB of LDS): small blocks
   // of which a compute unit holds several, each wave with one chunk in flight.
