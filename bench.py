@@ -294,10 +294,10 @@ def main() -> int:
                     v, _, _ = decode_run(args.batch, ctx, max(8, args.steps // 4), max(2, args.warmup // 4))
                     points[f"decode_b{args.batch}_ctx{ctx}"] = round(v, 1)
             # the 1B shape's workload (16 prompts of 64 to 4,096 tokens through the generation loop), with an
-            # engine of its own beside this one: what `--shape 1b` runs, with fewer steps
+            # engine of its own beside this one: what `--shape 1b` runs, with half the steps
             small = lq.LlamaConfig.from_dict(dict(CONFIG_1B))
             engine_1b = lq.random_engine(small, seed=0, dtype="bfloat16", max_tokens=16 * 8192, max_slots=16)
-            v, ms, ctx, line_1b = loop_run(engine_1b, small, 16, 64, 4096, max(16, args.steps // 2), max(4, args.warmup // 2))
+            v, ms, ctx, line_1b = loop_run(engine_1b, small, 16, 64, 4096, max(64, args.steps), max(8, args.warmup))
             bytes_1b = weight_bytes_per_step(small) + 16 * ctx * kv_bytes_per_token(small)
             points["decode_1b_b16"] = round(v, 1)
             points["decode_1b_b16_hbm_frac"] = round(bytes_1b / (ms * 1e-3) / 1e9 / HBM_GBPS, 4)

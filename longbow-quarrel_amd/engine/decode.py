@@ -79,7 +79,8 @@ class DecodeGraph:
         e = self.engine
         return e.make_context(self.ws, self.views[:7], self.slots or [0] * self.batch, [], [1] * self.batch,
                               self.bound, logits_out=self.logits,
-                              kernels=DryKernels(e.kernels) if dry else None, dry=dry, uneven=self.uneven)
+                              kernels=DryKernels(e.kernels) if dry else None, dry=dry, uneven=self.uneven,
+                              want_all=True)  # (views[7] lists the rows 0 .. batch - 1)
 
     def run_body(self, sampler: Sampler) -> None:
         """What one decoding step launches; the same calls whether captured or run directly."""

@@ -213,19 +213,21 @@ class Engine:
 
     def make_context(self, ws: Workspace, arrays: Sequence[torch.Tensor], slots: Sequence[int],
                      starts: Sequence[int], new: Sequence[int], max_len: int, logits_out=None, observe=None,
-                     kernels=None, dry: bool = False, uneven: bool = False) -> StepContext:
+                     kernels=None, dry: bool = False, uneven: bool = False, want_all: bool = False) -> StepContext:
         """The one place where a step's `StepContext` is put together, for direct and for captured steps.
         `arrays`: the device arrays tokens, row_seq, row_pos, seq_slot, seq_start, seq_len, cu_rows;
         `slots`, `starts`, `new`: per sequence, on the host (`starts` may be empty where the lengths
         live on the device only, as in a captured step); `max_len`: an upper bound of the lengths after
-        the step; `uneven`: whether a decoding step's sequences differ much in length (`Engine.lengths_uneven`)."""
+        the step; `uneven`: whether a decoding step's sequences differ much in length (`Engine.lengths_uneven`);
+        `want_all`: the logits of all the step's rows are wanted, in the rows' order."""
         tokens, row_seq, row_pos, seq_slot, seq_start, seq_len, cu_rows = arrays
         return StepContext(
             kernels=kernels if kernels is not None else self.kernels, dtype=self.dtype, device=self.device, ws=ws,
             rows=sum(new), batch=len(new), tokens=tokens, row_seq=row_seq, row_pos=row_pos, seq_slot=seq_slot,
             seq_start=seq_start, seq_len=seq_len, cu_rows=cu_rows, host_slots=list(slots), host_start=list(starts),
             host_new=list(new), max_new=max(new), max_len=max_len, decode=all(n == 1 for n in new),
-            logits_out=logits_out, observe=observe, dry=dry, uneven=uneven and all(n == 1 for n in new))
+            logits_out=logits_out, observe=observe, dry=dry, uneven=uneven and all(n == 1 for n in new),
+            want_all=want_all)
 
     def forward(self, ctx: StepContext, want_rows: torch.Tensor, n_want: int) -> Optional[torch.Tensor]:
         """The model over one step's rows, from this engine's cache."""
@@ -256,7 +258,8 @@ class Engine:
 
         self.ws.reset()
         ctx = self.make_context(self.ws, (d_tokens, d_row_seq, d_row_pos, d_slot, d_start, d_len, d_cu), slots,
-                                starts, new, max(lens), observe=observe, uneven=self.lengths_uneven(lens))
+                                starts, new, max(lens), observe=observe, uneven=self.lengths_uneven(lens),
+                                want_all=want_rows.size == rows and bool((want_rows == np.arange(rows)).all()))
         logits = self.forward(ctx, d_want, int(want_rows.size))
         cache.advance(growth)
         self.steps_run += 1

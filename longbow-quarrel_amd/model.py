@@ -20,7 +20,7 @@ from typing import Dict, List, Mapping, Optional, Sequence
 import torch
 
 from .parts.base import (BLOCKS, EMBEDDINGS, LOGIT_STEPS, MATRIX, NORMS, Block, BuildEnv, Embedding, LogitsStep, Norm,
-                         PartSpec, RowStats, StepContext, TensorSpec, build_part, project)
+                         NormedRows, PartSpec, RowStats, StepContext, TensorSpec, build_part, project, project_normed)
 
 
 @dataclass(frozen=True)
@@ -142,7 +142,10 @@ class DecoderModel:
                 cache = cache.read_only()
             block = self.blocks[run.layer]
             if block.takes_next_norm:
-                after = self.blocks[s.schedule[i + 1].layer].first_norm if i + 1 < len(s.schedule) else None
+                if i + 1 < len(s.schedule):
+                    after = self.blocks[s.schedule[i + 1].layer].first_norm
+                else:  # the final norm, where the head can take every row as it stands
+                    after = self.final_norm if ctx.want_all and n_want == ctx.rows else None
                 pending = block.forward(x, pending, ctx, cache, next_norm=after)
             else:
                 pending = block.forward(x, pending, ctx, cache)
@@ -151,13 +154,19 @@ class DecoderModel:
         if n_want == 0:
             return None
         ctx.ws.next_run()
-        picked = ctx.ws.alloc((n_want, s.width), torch.float32)
-        kn.gather_rows(x, want_rows, picked, delta=None if isinstance(pending, RowStats) else pending)
-        normed = self.final_norm.forward(picked, ctx)
         logits = ctx.logits_out
         if logits is None:
             logits = torch.empty((n_want, s.vocab_size), dtype=torch.float32, device=ctx.device)
-        project(kn, ctx, normed, self.head, logits)
+        # every row wanted as it stands, and the last block has left the final norm's statistics: the head
+        # applies the norm itself, without a kernel that picks rows and one that normalises them
+        folded = ctx.want_all and n_want == ctx.rows and isinstance(pending, RowStats) \
+            and pending.norm is self.final_norm \
+            and project_normed(kn, ctx, NormedRows(x, self.final_norm, pending), self.head, logits)
+        if not folded:
+            picked = ctx.ws.alloc((n_want, s.width), torch.float32)
+            kn.gather_rows(x, want_rows, picked, delta=None if isinstance(pending, RowStats) else pending)
+            normed = self.final_norm.forward(picked, ctx)
+            project(kn, ctx, normed, self.head, logits)
         if self.logits_step is not None:
             self.logits_step.forward(logits, ctx)
         return logits

@@ -254,6 +254,7 @@ class StepContext:
     # a decoding step whose sequences differ much in length (`Mixer.lengths_uneven`): a hint, which changes how the
     # attention kernel shares its work out and nothing in the result beyond the order of its sums
     uneven: bool = False
+    want_all: bool = False  # the logits of every row of the step are wanted, in the rows' order
     logits_out: Optional[torch.Tensor] = None  # where the logits go (a captured step's fixed buffer)
     # True while a step is only walked through to learn its workspace size: `kernels` then answers
     # size questions and launches nothing; a part that launches kernels of its own must not either

@@ -77,6 +77,31 @@ def test_chunked_prompts_and_mixed_steps(tmp_path):
     assert rel_err(o2[2], wb[89]) < TOL and rel_err(o3[0], wa[149]) < TOL
 
 
+def test_a_step_knows_when_every_row_is_wanted_in_order(tmp_path):
+    """`want_all` in the step's context (what lets the head take the stream's rows as they stand): set where
+    the wanted places are all the step's rows in their order, and only there."""
+    eng, ref = make(tmp_path, TINY_A)
+    seen = []
+    make_context = eng.make_context
+
+    def recording(*a, **k):
+        ctx = make_context(*a, **k)
+        seen.append(ctx.want_all)
+        return ctx
+
+    eng.make_context = recording
+    a, b = random_tokens(9, 256, 1), random_tokens(5, 256, 2)
+    wa, wb = ref.forward(a), ref.forward(b)
+    sa, sb = eng.new_sequence(), eng.new_sequence()
+    o = eng.step([StepEntry(sa, a[:4], range(4)), StepEntry(sb, b[:2], range(2))])  # all six rows
+    assert rel_err(o[:4], wa[:4]) < TOL and rel_err(o[4:], wb[:2]) < TOL
+    eng.step([StepEntry(sa, a[4:6], [1]), StepEntry(sb, b[2:4], [0, 1])])            # one row missing
+    eng.step([StepEntry(sa, a[6:8], [1, 0])])                                        # out of order
+    o = eng.step([StepEntry(sa, a[8:], [0]), StepEntry(sb, b[4:], [0])])             # a decoding step
+    assert rel_err(o[0], wa[8]) < TOL and rel_err(o[1], wb[4]) < TOL
+    assert seen == [True, False, False, True]
+
+
 def test_a_released_slot_leaves_no_trace(tmp_path):
     eng, ref = make(tmp_path, TINY_C, max_tokens=256)
     first = random_tokens(130, 331, 3)

@@ -303,7 +303,7 @@ def test_non_finite_logits_stop_generation_with_an_error(tmp_path_factory):
 WIDE = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 2176, "intermediate_size": 2312,
     "num_hidden_layers": 3, "num_attention_heads": 17, "num_key_value_heads": 1, "head_dim": 128,
-    "vocab_size": 1031, "max_position_embeddings": 512, "rms_norm_eps": 2e-6, "rope_theta": 40000.0,
+    "vocab_size": 2053, "max_position_embeddings": 512, "rms_norm_eps": 2e-6, "rope_theta": 40000.0,
     "rope_scaling": None, "tie_word_embeddings": False, "torch_dtype": "bfloat16",
     "bos_token_id": 1, "eos_token_id": 2,
 }
@@ -311,8 +311,9 @@ WIDE = {
 
 def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory):
     """A step of a few rows adds each projection's result into the stream in the projection itself
-    and leaves the norm to the projection that follows: against the plain implementation, as is the
-    same engine with these kernels switched off."""
+    and leaves the norm to the projection that follows (the final norm to the head, where every row's
+    logits are wanted): against the plain implementation, as is the same engine with these kernels
+    switched off."""
     folder = write_folder(tmp_path_factory.mktemp("wide"), WIDE, seed=3, std=0.03)
     eng = lq.load_engine(folder, dtype="bfloat16", max_tokens=1024)
     kn = eng.kernels
@@ -354,7 +355,7 @@ def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory
         kn.linear_residual, kn.linear_scaled = res, nrm
     layers = WIDE["num_hidden_layers"]
     steps = max(len(r) for r in reqs) - 5 + 1  # the prompts' step has 15 rows: few enough as well
-    assert calls["residual"] == 2 * layers * steps and calls["normed"] == (2 * layers - 1) * steps
+    assert calls["residual"] == 2 * layers * steps and calls["normed"] == 2 * layers * steps
     for got, w in zip(fused, want):
         assert rel_err(got, w) < TOL_BF16
     parts = kn.linear_fused_parts
