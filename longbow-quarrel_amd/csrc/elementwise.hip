@@ -19,10 +19,54 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
   for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = known ? to_f32(src[j]) : 0.0f;
 }
 
+// A bfloat16 row of a width that is a multiple of 8, 16 bytes a lane and load: all of a thread's loads are on
+// their way before its first store (the loop above waits for every element in turn: 9.4 us for a step's eight
+// rows of 4 096, this 4).
+typedef unsigned embed_u32x4 __attribute__((ext_vector_type(4)));
+typedef float embed_f32x4 __attribute__((ext_vector_type(4)));
+template <int PER_THREAD>
+__global__ __launch_bounds__(256) void embed_bf16_vec_kernel(const bf16_t* __restrict__ table,
+                                                             const int* __restrict__ tokens, float* __restrict__ out,
+                                                             int D, int vocab) {
+  const int r = blockIdx.x;
+  const long long tok = tokens[r];
+  const bool known = tok >= 0 && tok < vocab;
+  const embed_u32x4* src = (const embed_u32x4*)(table + (known ? tok : 0) * (long long)D);
+  embed_f32x4* dst = (embed_f32x4*)(out + (long long)r * D);
+  const int chunks = D / 8;
+  embed_u32x4 v[PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < PER_THREAD; ++i) {
+    const int c = threadIdx.x + i * 256;
+    v[i] = (c < chunks && known) ? src[c] : (embed_u32x4){0u, 0u, 0u, 0u};
+  }
+#pragma unroll
+  for (int i = 0; i < PER_THREAD; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < chunks) {
+      dst[2 * c] = (embed_f32x4){__uint_as_float(v[i][0] << 16), __uint_as_float(v[i][0] & 0xffff0000u),
+                                 __uint_as_float(v[i][1] << 16), __uint_as_float(v[i][1] & 0xffff0000u)};
+      dst[2 * c + 1] = (embed_f32x4){__uint_as_float(v[i][2] << 16), __uint_as_float(v[i][2] & 0xffff0000u),
+                                     __uint_as_float(v[i][3] << 16), __uint_as_float(v[i][3] & 0xffff0000u)};
+    }
+  }
+}
+
 extern "C" int lq_embed(const void* table, int table_dtype, const int* tokens, float* out, int rows,
                         int D, int vocab, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && D > 0 && vocab > 0, "embed: rows %d, width %d and table rows %d must be positive", rows, D, vocab);
   const int threads = D >= 1024 ? 256 : 64;
+  if (table_dtype == LQ_BF16 && D % 8 == 0 && D >= 2048 && D <= 8 * 256 * 8 && (uintptr_t)table % 16 == 0 &&
+      (uintptr_t)out % 16 == 0) {
+    if (D <= 8 * 256 * 2)
+      embed_bf16_vec_kernel<2><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab);
+    else if (D <= 8 * 256 * 4)
+      embed_bf16_vec_kernel<4><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab);
+    else
+      embed_bf16_vec_kernel<8><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab);
+    LQ_CHECK_LAUNCH("embed");
+    return 0;
+  }
   if (table_dtype == LQ_F32)
     embed_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, tokens, out, D, vocab);
   else if (table_dtype == LQ_BF16)

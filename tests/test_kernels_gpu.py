@@ -32,7 +32,7 @@ def i32(values):
 # --------------------------------------------------------------------------- rows
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width", [331, 4096])
+@pytest.mark.parametrize("width", [331, 2048, 2176, 4096, 5000, 8192, 16384, 16392])
 def test_embed(kn, dtype, width):
     table = rnd((97, width), 1, dtype)
     toks = i32([5, 96, 0, 5, 33])
