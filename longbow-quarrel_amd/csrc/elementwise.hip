@@ -551,6 +551,117 @@ __global__ __launch_bounds__(256) void rope_store_vec_kernel(
   }
 }
 
+// The same from the float32 pieces that a product leaves where it shares K over blocks (`pieces` partial sums,
+// `piece_stride` elements apart, each with q, k and v side by side in rows of ld elements): a thread adds the
+// pieces of its 8 values up in ascending order, rounds the sums to bfloat16 as the whole product would have,
+// and goes on as above; the rotated q goes to a buffer of its own.
+__device__ inline u32x4_t sum_pieces8(const float* p, int pieces, long long piece_stride) {
+  typedef float f32x4_t __attribute__((ext_vector_type(4)));
+  f32x4_t lo = *(const f32x4_t*)p, hi = *(const f32x4_t*)(p + 4);
+  // four pieces are asked for together (one round trip to memory, not four) and added in their order
+  for (int s0 = 1; s0 < pieces; s0 += 4) {
+    f32x4_t tl[4], th[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const long long at = (long long)min(s0 + j, pieces - 1) * piece_stride;
+      tl[j] = *(const f32x4_t*)(p + at);
+      th[j] = *(const f32x4_t*)(p + at + 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (s0 + j < pieces) {
+        lo += tl[j];
+        hi += th[j];
+      }
+    }
+  }
+  u32x4_t r;
+  r[0] = (unsigned)f32_to_bf16(lo[0]).bits | ((unsigned)f32_to_bf16(lo[1]).bits << 16);
+  r[1] = (unsigned)f32_to_bf16(lo[2]).bits | ((unsigned)f32_to_bf16(lo[3]).bits << 16);
+  r[2] = (unsigned)f32_to_bf16(hi[0]).bits | ((unsigned)f32_to_bf16(hi[1]).bits << 16);
+  r[3] = (unsigned)f32_to_bf16(hi[2]).bits | ((unsigned)f32_to_bf16(hi[3]).bits << 16);
+  return r;
+}
+
+__global__ __launch_bounds__(256) void rope_store_pieces_kernel(
+    const float* __restrict__ qkv, int ld, int pieces, long long piece_stride, bf16_t* __restrict__ q_out, int ldq,
+    int nh, int nkv, int hd, const double* __restrict__ freqs, const int* __restrict__ row_pos,
+    const int* __restrict__ row_seq, const int* __restrict__ seq_slot, const int* __restrict__ block_table,
+    int bt_stride, bf16_t* __restrict__ kcache, bf16_t* __restrict__ vcache, int BS) {
+  extern __shared__ float cs[];  // cos[hd/2], sin[hd/2]
+  const int r = blockIdx.x;
+  const int half = hd / 2, hv = half / 8;
+  const int p = row_pos[r];
+  const long long blk = block_table[(long long)seq_slot[row_seq[r]] * bt_stride + p / BS];
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const double a = (double)p * freqs[i];
+    const double n = rint(a * 0.15915494309189533577);
+    double rem = fma(-n, 6.283185307179586232, a);
+    rem = fma(-n, 2.4492935982947064e-16, rem);
+    float sn, c;
+    sincosf((float)rem, &sn, &c);
+    cs[i] = c;
+    cs[half + i] = sn;
+  }
+  __syncthreads();
+  const float* qr = qkv + (long long)r * ld;
+  const float* kr = qr + nh * hd;
+  const float* vr = kr + nkv * hd;
+  bf16_t* qo = q_out + (long long)r * ldq;
+  for (int idx = threadIdx.x; idx < nh * hv; idx += blockDim.x) {
+    const int h = idx / hv, i = (idx - h * hv) * 8;
+    u32x4_t a = sum_pieces8(qr + h * hd + i, pieces, piece_stride);
+    u32x4_t b = sum_pieces8(qr + h * hd + half + i, pieces, piece_stride);
+    rotate8(a, b, cs + i, cs + half + i);
+    *(u32x4_t*)(qo + h * hd + i) = a;
+    *(u32x4_t*)(qo + h * hd + half + i) = b;
+  }
+  const int off = p % BS;
+  for (int idx = threadIdx.x; idx < nkv * hv; idx += blockDim.x) {
+    const int h = idx / hv, i = (idx - h * hv) * 8;
+    u32x4_t a = sum_pieces8(kr + h * hd + i, pieces, piece_stride);
+    u32x4_t b = sum_pieces8(kr + h * hd + half + i, pieces, piece_stride);
+    rotate8(a, b, cs + i, cs + half + i);
+    bf16_t* dst = kcache + ((blk * nkv + h) * BS + off) * (long long)hd;
+    *(u32x4_t*)(dst + i) = a;
+    *(u32x4_t*)(dst + half + i) = b;
+  }
+  for (int idx = threadIdx.x; idx < nkv * 2 * hv; idx += blockDim.x) {
+    const int h = idx / (2 * hv), d = (idx - h * 2 * hv) * 8;
+    const u32x4_t x = sum_pieces8(vr + h * hd + d, pieces, piece_stride);
+    bf16_t* dst = vcache + ((blk * nkv + h) * hd + d) * (long long)BS + off;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      bf16_t lo, hi;
+      lo.bits = (uint16_t)(x[j] & 0xffffu);
+      hi.bits = (uint16_t)(x[j] >> 16);
+      dst[(long long)(2 * j) * BS] = lo;
+      dst[(long long)(2 * j + 1) * BS] = hi;
+    }
+  }
+}
+
+extern "C" int lq_rope_store_pieces(const float* qkv, int ld, int pieces, long long piece_stride, void* q_out, int ldq,
+                                    int rows, int nh, int nkv, int hd, const double* freqs, const int* row_pos,
+                                    const int* row_seq, const int* seq_slot, const int* block_table, int bt_stride,
+                                    void* kcache, void* vcache, int block_size, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && pieces >= 1, "rope_store (pieces): rows %d, pieces %d", rows, pieces);
+  LQ_REQUIRE(hd > 0 && hd % 16 == 0 && nh > 0 && nkv > 0, "rope_store (pieces): head size %d, heads %d / %d", hd, nh, nkv);
+  LQ_REQUIRE(ld >= (nh + 2 * nkv) * hd && ldq >= nh * hd && ld % 4 == 0 && ldq % 8 == 0 && piece_stride % 4 == 0 &&
+                 (pieces == 1 || piece_stride >= (long long)rows * ld),
+             "rope_store (pieces): row strides %d / %d, piece stride %lld", ld, ldq, piece_stride);
+  LQ_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)q_out % 16) == 0 && ((uintptr_t)kcache % 16) == 0,
+             "rope_store (pieces): rows and caches must be 16-byte aligned");
+  LQ_REQUIRE(block_size > 0 && bt_stride > 0, "rope_store: block size %d, table stride %d", block_size, bt_stride);
+  LQ_REQUIRE(qkv && q_out && freqs && row_pos && row_seq && seq_slot && block_table && kcache && vcache,
+             "rope_store (pieces): null argument");
+  rope_store_pieces_kernel<<<rows, 256, (size_t)hd * sizeof(float), stream>>>(
+      qkv, ld, pieces, piece_stride, (bf16_t*)q_out, ldq, nh, nkv, hd, freqs, row_pos, row_seq, seq_slot, block_table,
+      bt_stride, (bf16_t*)kcache, (bf16_t*)vcache, block_size);
+  LQ_CHECK_LAUNCH("rope_store (pieces)");
+  return 0;
+}
+
 // The same for the rows of prompts, eight positions at a time: a block takes the rows of one sequence whose
 // positions lie in one group [8 g, 8 g + 8), so that the values of a whole group go into the transposed V
 // cache as runs of eight positions (16 bytes) instead of two bytes at a time, and takes cos and sin from

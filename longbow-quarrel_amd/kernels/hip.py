@@ -20,7 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
-ABI_VERSION = 3  # lq_abi_version() of the library these wrappers were written for
+ABI_VERSION = 4  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -350,6 +350,46 @@ class HipKernels:
         reads it takes eight positions a workgroup and pays from about a thousand rows on (19 against 22 us at
         2 048 rows and 49 against 74 at 8 192, but 8.7 against 7.1 us at 128 rows)."""
         return rows >= 1024
+
+    @query
+    def rope_store_adds_pieces(self, dtype: torch.dtype, rows: int, heads: int, kv_heads: int, head_dim: int) -> bool:
+        """Whether `rope_store_pieces` takes q, k and v of such a step as the float32 pieces of a product
+        that shares K over blocks (`linear_pieces`): bfloat16 steps of fewer rows than `rope_store` wants a
+        table for, head sizes in steps of 16."""
+        return (not self.force_generic and dtype == torch.bfloat16 and head_dim % 16 == 0
+                and not self.rope_store_takes_table(rows))
+
+    def rope_store_pieces(self, qkv: torch.Tensor, q_out: torch.Tensor, heads: int, kv_heads: int, head_dim: int,
+                          freqs: torch.Tensor, row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor,
+                          block_table: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_size: int) -> None:
+        """`rope_store` for qkv float32 [pieces, rows, (heads + 2 kv_heads) * head_dim], the partial sums of
+        the projection with q, k and v side by side: adds the pieces in ascending order, rounds the sums to
+        bfloat16 as the whole product would have, rotates q (into q_out, bfloat16 [rows, heads * head_dim])
+        and k, and writes k and v into the paged cache."""
+        self._dev(qkv, q_out, freqs, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
+        if qkv.dim() != 3 or qkv.dtype != torch.float32 or not qkv.is_contiguous() \
+                or qkv.shape[2] != (heads + 2 * kv_heads) * head_dim:
+            raise KernelLibraryError("rope_store_pieces: qkv must be dense float32 [pieces, rows, (heads + 2 kv_heads) * head_dim]")
+        pieces, rows, width = qkv.shape
+        if q_out.dtype != torch.bfloat16 or tuple(q_out.shape) != (rows, heads * head_dim) \
+                or kcache.dtype != torch.bfloat16 or vcache.dtype != torch.bfloat16:
+            raise KernelLibraryError("rope_store_pieces: q_out bfloat16 [rows, heads * head_dim], bfloat16 caches")
+        self._i32(row_pos, "row_pos", rows)
+        self._i32(row_seq, "row_seq", rows)
+        if freqs.dtype != torch.float64 or freqs.numel() != head_dim // 2 or not freqs.is_contiguous():
+            raise KernelLibraryError(f"rope_store_pieces: freqs must be float64 of {head_dim // 2} entries")
+        if seq_slot.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.dim() != 2:
+            raise KernelLibraryError("rope_store_pieces: seq_slot and block_table must be int32 (table 2-D)")
+        nb = kcache.shape[0]
+        if tuple(kcache.shape) != (nb, kv_heads, block_size, head_dim) or \
+                tuple(vcache.shape) != (nb, kv_heads, head_dim, block_size) or \
+                not kcache.is_contiguous() or not vcache.is_contiguous():
+            raise KernelLibraryError("rope_store_pieces: cache tensors do not have the paged layout")
+        self._check(self.lib.lq_rope_store_pieces(
+            _ptr(qkv), c_int(width), c_int(pieces), c_longlong(qkv.stride(0)), _ptr(q_out),
+            c_int(self._rows2d(q_out, "q_out")), c_int(rows), c_int(heads), c_int(kv_heads), c_int(head_dim),
+            _ptr(freqs), _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(block_table),
+            c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size), self.stream))
 
     def rope_store(self, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
                    heads: int, kv_heads: int, head_dim: int, freqs: Optional[torch.Tensor],

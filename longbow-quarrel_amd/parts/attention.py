@@ -76,6 +76,21 @@ class GQAttention(Mixer):
         ask = getattr(kernels, "decode_lengths_uneven", None)
         return bool(ask(lengths)) if ask is not None and self.window == 0 else False
 
+    def _rotate_and_store(self, q, k, v, freqs, ctx: StepContext, cache: LayerCache) -> None:
+        kn = ctx.kernels
+        if freqs is None:
+            self.position.apply(q, k, ctx)
+        if cache.write:
+            # the step's table of cos and sin, where the position encoding keeps one (the same for every layer)
+            by_groups = getattr(kn, "rope_store_takes_table", lambda rows: False)(q.shape[0])
+            table = self.position.cos_sin(ctx) if (by_groups and freqs is not None
+                                                   and hasattr(self.position, "cos_sin")) else None
+            kn.rope_store(q, k, v, self.heads, self.kv_heads, self.head_dim, freqs, ctx.row_pos,
+                          ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size,
+                          cos_sin=table, cu_rows=ctx.cu_rows if table is not None else None)
+        elif freqs is not None:
+            kn.rope_store(q, None, None, self.heads, 0, self.head_dim, freqs, ctx.row_pos)
+
     def forward(self, h, ctx: StepContext, cache: Optional[LayerCache], sink=None) -> Optional[torch.Tensor]:
         if cache is None or cache.k is None:
             raise RuntimeError("attention needs a key/value cache")
@@ -93,7 +108,24 @@ class GQAttention(Mixer):
         if (folded and not isinstance(h, NormedRows) and self.w_qkv.dtype == h.dtype
                 and getattr(kn, "attention_adds_pieces", lambda *a: False)(*shape)):
             pieces = kn.linear_pieces(h.dtype, rows, width, self.width)
-        if pieces > 1:
+        # A step of a few dozen to a few hundred rows that writes the cache through `rope_store`: the same, with
+        # the pieces added up by the kernel that rotates (its columns alone would leave most of the chip idle,
+        # every block reading all the rows).
+        stored_pieces = False
+        if (pieces == 1 and not folded and cache.write and freqs is not None and not isinstance(h, NormedRows)
+                and self.w_qkv.dtype == h.dtype
+                and getattr(kn, "rope_store_adds_pieces", lambda *a: False)(ctx.dtype, rows, self.heads, self.kv_heads,
+                                                                            self.head_dim)):
+            pieces = kn.linear_pieces(h.dtype, rows, width, self.width)
+            stored_pieces = pieces > 1
+        if stored_pieces:
+            qkv = ctx.ws.alloc((pieces, rows, width), torch.float32)
+            project(kn, ctx, h, self.w_qkv, qkv)
+            q = ctx.ws.alloc((rows, self.q_width), ctx.dtype)
+            kn.rope_store_pieces(qkv, q, self.heads, self.kv_heads, self.head_dim, freqs, ctx.row_pos, ctx.row_seq,
+                                 ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size)
+            k = v = None
+        elif pieces > 1:
             qkv = ctx.ws.alloc((pieces, rows, width), torch.float32)
             project(kn, ctx, h, self.w_qkv, qkv)
             first, stride = qkv[0], qkv.stride(0)
@@ -104,9 +136,10 @@ class GQAttention(Mixer):
                 if isinstance(h, NormedRows):
                     h = h.tensor(ctx)
                 project(kn, ctx, h, self.w_qkv, qkv)
-        q = first[:, : self.q_width]
-        k = first[:, self.q_width : self.q_width + self.kv_width]
-        v = first[:, self.q_width + self.kv_width :]
+        if not stored_pieces:
+            q = first[:, : self.q_width]
+            k = first[:, self.q_width : self.q_width + self.kv_width]
+            v = first[:, self.q_width + self.kv_width :]
         att = ctx.ws.alloc((rows, self.q_width), ctx.dtype)
         need = kn.attention_workspace(ctx.dtype, rows, self.heads, self.kv_heads, self.head_dim,
                                       cache.block_size, ctx.decode, ctx.max_len)
@@ -118,18 +151,8 @@ class GQAttention(Mixer):
                          self.scale, self.window, decode=True, max_len=ctx.max_len, workspace=scratch,
                          k_new=k, v_new=v, cos_sin=self.position.cos_sin(ctx), uneven=ctx.uneven, **more)
         else:
-            if freqs is None:
-                self.position.apply(q, k, ctx)
-            if cache.write:
-                # the step's table of cos and sin, where the position encoding keeps one (the same for every layer)
-                by_groups = getattr(kn, "rope_store_takes_table", lambda rows: False)(q.shape[0])
-                table = self.position.cos_sin(ctx) if (by_groups and freqs is not None
-                                                       and hasattr(self.position, "cos_sin")) else None
-                kn.rope_store(q, k, v, self.heads, self.kv_heads, self.head_dim, freqs, ctx.row_pos,
-                              ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size,
-                              cos_sin=table, cu_rows=ctx.cu_rows if table is not None else None)
-            elif freqs is not None:
-                kn.rope_store(q, None, None, self.heads, 0, self.head_dim, freqs, ctx.row_pos)
+            if not stored_pieces:  # (else q is rotated and the cache written already)
+                self._rotate_and_store(q, k, v, freqs, ctx, cache)
             kn.attention(q, att, self.heads, self.kv_heads, self.head_dim, ctx.row_pos, ctx.row_seq,
                          ctx.seq_slot, ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size,
                          self.scale, self.window, decode=ctx.decode, max_len=ctx.max_len, workspace=scratch,

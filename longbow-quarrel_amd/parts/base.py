@@ -169,7 +169,7 @@ class _Arena:
         n = 1
         for s in shape:
             n *= int(s)
-        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        nbytes = n * dtype.itemsize
         start = (self.off + self.ALIGN - 1) // self.ALIGN * self.ALIGN
         end = start + nbytes
         self.off = end

@@ -683,6 +683,43 @@ def test_rope_store_by_groups_of_eight_positions_writes_the_same_bits(kn, heads,
     assert bool((vc.cpu().permute(0, 3, 1, 2)[~touched] == 3.0).all())
 
 
+@pytest.mark.parametrize("heads,kv_heads,hd,pieces", [(32, 8, 128, 4), (6, 3, 48, 3), (8, 2, 64, 1), (3, 1, 16, 7)])
+def test_rope_store_from_the_pieces_of_a_product_writes_the_same_bits(kn, heads, kv_heads, hd, pieces):
+    """q, k and v as the float32 partial sums that a product leaves where it shares K over blocks: the kernel
+    adds them in ascending order, rounds the sums to bfloat16 and rotates and stores as `rope_store` does with
+    rows that were summed and rounded beforehand; q, the K cache and the V cache come out bit for bit the same."""
+    freqs = plain.rope_frequencies(hd, 500000.0).to(DEV)
+    starts, lens = [0, 3, 64, 70], [130, 1, 9, 60]
+    slots = [4, 2, 7, 1]
+    n_blocks, per_seq = 40, 4
+    g = torch.Generator().manual_seed(10)
+    table = torch.randperm(n_blocks, generator=g)[: 8 * per_seq].view(8, per_seq).to(torch.int32).to(DEV)
+    pos, row_seq = [], []
+    for b, (st, n) in enumerate(zip(starts, lens)):
+        pos += list(range(st, st + n))
+        row_seq += [b] * n
+    rows = len(pos)
+    width = (heads + 2 * kv_heads) * hd
+    parts = rnd((pieces, rows, width), 34, torch.float32)
+    total = parts[0].clone()
+    for s in range(1, pieces):
+        total = total + parts[s]
+    qkv = total.bfloat16()
+    caches = []
+    for _ in range(2):
+        caches.append((torch.full((n_blocks, kv_heads, BS, hd), 3.0, dtype=torch.bfloat16, device=DEV),
+                       torch.full((n_blocks, kv_heads, hd, BS), 3.0, dtype=torch.bfloat16, device=DEV)))
+    q, k = qkv[:, : heads * hd], qkv[:, heads * hd : (heads + kv_heads) * hd]
+    v = qkv[:, (heads + kv_heads) * hd :]
+    kn.rope_store(q, k, v, heads, kv_heads, hd, freqs, i32(pos), i32(row_seq), i32(slots), table, caches[0][0],
+                  caches[0][1], BS)
+    q_out = torch.empty((rows, heads * hd), dtype=torch.bfloat16, device=DEV)
+    kn.rope_store_pieces(parts, q_out, heads, kv_heads, hd, freqs, i32(pos), i32(row_seq), i32(slots), table,
+                         caches[1][0], caches[1][1], BS)
+    assert torch.equal(q_out, q)
+    assert torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
+
+
 @pytest.mark.parametrize("head_dim,heads,kv_heads,lengths", [
     (128, 8, 2, [5000, 300, 40, 1025, 256, 257, 2, 3000]),            # one long sequence among short ones
     (64, 4, 1, [700, 64, 1, 1500, 1500, 513, 30, 31, 32, 33, 9000]),  # one kv head; 11 sequences
