@@ -149,10 +149,15 @@ class _Arena:
 
     def __init__(self, device: torch.device, nbytes: int) -> None:
         self.device = device
-        self.buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
         self.off = 0
         self.high = 0
         self._spill: List[torch.Tensor] = []
+        self._set_buffer(nbytes)
+
+    def _set_buffer(self, nbytes: int) -> None:
+        nbytes = (int(nbytes) + self.ALIGN - 1) // self.ALIGN * self.ALIGN
+        self.buf = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        self._typed = {}  # dtype -> the whole buffer seen as that dtype: a piece of it is one view away
 
     def rewind(self) -> None:
         self.off = 0
@@ -160,7 +165,7 @@ class _Arena:
 
     def reset(self, grow: bool) -> None:
         if self.high > self.buf.numel() and grow:
-            self.buf = torch.empty(int(self.high * 1.25) + self.ALIGN, dtype=torch.uint8, device=self.device)
+            self._set_buffer(int(self.high * 1.25) + self.ALIGN)
         self.off = 0
         self.high = 0
         self._spill = []
@@ -180,7 +185,15 @@ class _Arena:
             t = torch.empty(tuple(shape), dtype=dtype, device=self.device)  # this step only; reset() grows
             self._spill.append(t)
             return t
-        return self.buf[start:end].view(dtype).view(tuple(shape))
+        base = self._typed.get(dtype)
+        if base is None:
+            base = self._typed[dtype] = self.buf.view(dtype)
+        shape = tuple(shape)
+        strides, step = [], 1
+        for d in reversed(shape):
+            strides.append(step)
+            step *= int(d)
+        return base.as_strided(shape, strides[::-1], start // dtype.itemsize)
 
 
 class Workspace:
