@@ -51,6 +51,16 @@ def load_library() -> ctypes.CDLL:
     if lib.lq_abi_version() != ABI_VERSION:
         raise KernelLibraryError(f"{path} speaks version {lib.lq_abi_version()} of the kernel interface, "
                                  f"this package version {ABI_VERSION}: build it again")
+    # The entry points that a prompt step calls most take plain Python numbers (declared argument types
+    # save making a ctypes object for each of them: a call from Python is 5 us instead of 10, where the
+    # launch itself is 3).
+    vp, ci, cl, cf = c_void_p, c_int, c_longlong, c_float
+    lib.lq_linear.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cl, ci, vp]
+    lib.lq_linear_swiglu.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp]
+    lib.lq_rmsnorm.argtypes = [vp, vp, ci, ci, cl, vp, cf, vp, ci, ci, ci, vp]
+    lib.lq_attention.argtypes = [vp, ci, vp, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, vp, vp, ci, vp, vp, ci, cf, ci, ci, ci,
+                                 vp, cl, vp, cl, vp, vp, ci, ci, vp, ci, ci, cl, ci, vp]
+    lib.lq_rope_store_pieces.argtypes = [vp, ci, ci, cl, vp, ci, ci, ci, ci, ci, vp, vp, vp, vp, vp, ci, vp, vp, ci, vp]
     _LIB = lib
     return lib
 
@@ -133,6 +143,20 @@ class HipKernels:
                 raise KernelLibraryError("kernel arguments must be contiguous in their last dimension")
 
     @staticmethod
+    def _mat(t: torch.Tensor, what: str):
+        """(rows, columns, row stride in elements) of a 2-D tensor on the GPU whose rows are dense: `_dev` and
+        `_rows2d` in one pass."""
+        sh = t.shape
+        if len(sh) != 2:
+            raise KernelLibraryError(f"{what}: expected a 2-D tensor, found shape {tuple(sh)}")
+        if not t.is_cuda:
+            raise KernelLibraryError("kernel arguments must live on the GPU")
+        st = t.stride()
+        if st[1] != 1 and sh[1] != 1:
+            raise KernelLibraryError("kernel arguments must be contiguous in their last dimension")
+        return sh[0], sh[1], (st[0] if sh[0] > 1 else max(st[0], sh[1]))
+
+    @staticmethod
     def _rows2d(t: torch.Tensor, what: str) -> int:
         """Row stride in elements of a 2-D view whose last dimension is dense."""
         if t.dim() != 2:
@@ -170,19 +194,22 @@ class HipKernels:
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
                 delta: Optional[torch.Tensor] = None) -> None:
         """(x += delta;) out = x / sqrt(mean(x^2) + eps) * weight, row by row; x is float32."""
-        self._dev(x, weight, out, delta)
+        rows, width, ldx = self._mat(x, "rmsnorm: x")
+        if delta is not None:
+            self._dev(delta)
         pieces, stride = self._pieces(delta, x, "rmsnorm")
-        rows, width = x.shape
-        if x.dtype != torch.float32 or not x.is_contiguous():
+        if x.dtype != torch.float32 or (ldx != width and rows > 1):
             raise KernelLibraryError("rmsnorm: x must be dense float32")
-        if weight.dtype != torch.float32 or weight.numel() != width or not weight.is_contiguous():
+        if weight.dtype != torch.float32 or weight.numel() != width or not weight.is_contiguous() or not weight.is_cuda:
             raise KernelLibraryError(f"rmsnorm: weight must be float32 of {width} entries")
-        if tuple(out.shape) != (rows, width) or not out.is_contiguous():
+        ro, wo, ldo = self._mat(out, "rmsnorm: out")
+        if ro != rows or wo != width or (ldo != width and rows > 1):
             raise KernelLibraryError("rmsnorm: out must be dense and shaped like x")
-        self._check(self.lib.lq_rmsnorm(_ptr(x), _ptr(delta), c_int(_code(delta) if delta is not None else 0),
-                                        c_int(pieces), c_longlong(stride),
-                                        _ptr(weight), c_float(eps), _ptr(out), c_int(_code(out)),
-                                        c_int(rows), c_int(width), self.stream))
+        rc = self.lib.lq_rmsnorm(x.data_ptr(), 0 if delta is None else delta.data_ptr(),
+                                 _code(delta) if delta is not None else 0, pieces, stride, weight.data_ptr(),
+                                 float(eps), out.data_ptr(), _code(out), rows, width, self.stream)
+        if rc:
+            self._check(rc)
 
     def add(self, x: torch.Tensor, delta: torch.Tensor) -> None:
         """x += delta (x float32)."""
@@ -214,27 +241,26 @@ class HipKernels:
     def linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
         """out[M, N] = x[M, K] . w[N, K]^T with 32-bit accumulation; or out[pieces, M, N] with
         `linear_pieces` pieces that sum to it."""
-        self._dev(x, w, out)
-        if x.dim() != 2 or w.dim() != 2 or out.dim() not in (2, 3):
-            raise KernelLibraryError("linear: 2-D tensors are needed")
-        m, k = x.shape
-        n = w.shape[0]
-        if w.shape[1] != k or tuple(out.shape[-2:]) != (m, n):
+        m, k, ldx = self._mat(x, "linear: x")
+        n, kw, ldw = self._mat(w, "linear: w")
+        pieces, stride = 1, 0
+        if out.dim() == 3:
+            pieces, stride = out.shape[0], m * n
+            if not out.is_cuda or not out.is_contiguous() or pieces != self.linear_pieces(x.dtype, m, n, k):
+                raise KernelLibraryError(f"linear: {pieces} pieces asked (dense, on the GPU), linear_pieces says "
+                                         f"{self.linear_pieces(x.dtype, m, n, k)}")
+            mo, no, ldc = out.shape[1], out.shape[2], n
+        else:
+            mo, no, ldc = self._mat(out, "linear: out")
+        if kw != k or mo != m or no != n:
             raise KernelLibraryError(
                 f"linear: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
         if x.dtype != w.dtype:
             raise KernelLibraryError(f"linear: x is {x.dtype} but w is {w.dtype}")
-        pieces, stride = 1, 0
-        if out.dim() == 3:
-            pieces, stride = out.shape[0], m * n
-            if not out.is_contiguous() or pieces != self.linear_pieces(x.dtype, m, n, k):
-                raise KernelLibraryError(f"linear: {pieces} pieces asked, linear_pieces says "
-                                         f"{self.linear_pieces(x.dtype, m, n, k)}")
-        ldc = self._rows2d(out[0], "out") if out.dim() == 3 else self._rows2d(out, "out")
-        self._check(self.lib.lq_linear(_ptr(x), _ptr(w), _ptr(out), c_int(_code(x)), c_int(_code(out)),
-                                       c_int(m), c_int(n), c_int(k), c_int(self._rows2d(x, "x")),
-                                       c_int(self._rows2d(w, "w")), c_int(ldc), c_int(pieces), c_longlong(stride),
-                                       c_int(1 if self.force_generic else 0), self.stream))
+        rc = self.lib.lq_linear(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(x), _code(out), m, n, k, ldx, ldw,
+                                ldc, pieces, stride, 1 if self.force_generic else 0, self.stream)
+        if rc:
+            self._check(rc)
 
     # -- the two products around a norm, for a few rows (decoding): x += act . w^T leaves every row's
     # sum of squares in parts, and the product after the norm normalises its input from them itself
@@ -300,18 +326,16 @@ class HipKernels:
         """out[M, I] = silu(gate) * up with [gate | up] = x . w^T, in one kernel.  w [2 I, K] holds the
         gate and up rows interleaved in groups of 8: rows 16j..16j+7 gate 8j..8j+7, rows 16j+8..16j+15
         up 8j..8j+7 (see `interleave_gate_up`)."""
-        self._dev(x, w, out)
-        if x.dim() != 2 or w.dim() != 2 or out.dim() != 2:
-            raise KernelLibraryError("linear_swiglu: 2-D tensors are needed")
-        m, k = x.shape
-        n = w.shape[0]
-        if w.shape[1] != k or tuple(out.shape) != (m, n // 2) or n % 16 != 0 or x.dtype != w.dtype:
+        m, k, ldx = self._mat(x, "linear_swiglu: x")
+        n, kw, ldw = self._mat(w, "linear_swiglu: w")
+        mo, no, ldc = self._mat(out, "linear_swiglu: out")
+        if kw != k or mo != m or no != n // 2 or n % 16 != 0 or x.dtype != w.dtype:
             raise KernelLibraryError(
                 f"linear_swiglu: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
-        self._check(self.lib.lq_linear_swiglu(_ptr(x), _ptr(w), _ptr(out), c_int(_code(x)), c_int(_code(out)),
-                                              c_int(m), c_int(n), c_int(k), c_int(self._rows2d(x, "x")),
-                                              c_int(self._rows2d(w, "w")), c_int(self._rows2d(out, "out")),
-                                              self.stream))
+        rc = self.lib.lq_linear_swiglu(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(x), _code(out), m, n, k,
+                                       ldx, ldw, ldc, self.stream)
+        if rc:
+            self._check(rc)
 
     @staticmethod
     def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
@@ -385,11 +409,13 @@ class HipKernels:
                 tuple(vcache.shape) != (nb, kv_heads, head_dim, block_size) or \
                 not kcache.is_contiguous() or not vcache.is_contiguous():
             raise KernelLibraryError("rope_store_pieces: cache tensors do not have the paged layout")
-        self._check(self.lib.lq_rope_store_pieces(
-            _ptr(qkv), c_int(width), c_int(pieces), c_longlong(qkv.stride(0)), _ptr(q_out),
-            c_int(self._rows2d(q_out, "q_out")), c_int(rows), c_int(heads), c_int(kv_heads), c_int(head_dim),
-            _ptr(freqs), _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(block_table),
-            c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size), self.stream))
+        rc = self.lib.lq_rope_store_pieces(
+            qkv.data_ptr(), width, pieces, qkv.stride(0), q_out.data_ptr(), self._rows2d(q_out, "q_out"), rows, heads,
+            kv_heads, head_dim, freqs.data_ptr(), row_pos.data_ptr(), row_seq.data_ptr(), seq_slot.data_ptr(),
+            block_table.data_ptr(), int(block_table.stride(0)), kcache.data_ptr(), vcache.data_ptr(), block_size,
+            self.stream)
+        if rc:
+            self._check(rc)
 
     def rope_store(self, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
                    heads: int, kv_heads: int, head_dim: int, freqs: Optional[torch.Tensor],
@@ -564,16 +590,15 @@ class HipKernels:
                 raise KernelLibraryError("attention: cos_sin must be dense float32 [rows, head_dim/2, 2]")
             ldk, ldv = self._rows2d(k_new, "k_new"), self._rows2d(v_new, "v_new")
         tickets = self.tickets(q.device)
+        folds = cos_sin is not None
         rc = self.lib.lq_attention(
-            _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")),
-            c_int(_code(out)), c_int(rows), c_int(batch), c_int(heads), c_int(kv_heads), c_int(head_dim),
-            _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot), _ptr(cu_rows), _ptr(block_table),
-            c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
-            c_float(scale), c_int(window), c_int(1 if decode else 0), c_int(max_len), _ptr(workspace),
-            c_longlong(ws_n), _ptr(tickets), c_longlong(tickets.numel()), _ptr(k_new if cos_sin is not None else None),
-            _ptr(v_new if cos_sin is not None else None), c_int(ldk), c_int(ldv), _ptr(cos_sin),
-            c_int(1 if uneven and decode else 0), c_int(pieces), c_longlong(piece_stride),
-            c_int(1 if self.force_generic else 0), self.stream)
+            q.data_ptr(), self._rows2d(q, "q"), out.data_ptr(), self._rows2d(out, "out"), _code(out), rows, batch,
+            heads, kv_heads, head_dim, row_pos.data_ptr(), row_seq.data_ptr(), seq_slot.data_ptr(), cu_rows.data_ptr(),
+            block_table.data_ptr(), int(block_table.stride(0)), kcache.data_ptr(), vcache.data_ptr(), block_size,
+            float(scale), window, 1 if decode else 0, max_len, 0 if workspace is None else workspace.data_ptr(), ws_n,
+            tickets.data_ptr(), tickets.numel(), k_new.data_ptr() if folds else 0, v_new.data_ptr() if folds else 0,
+            ldk, ldv, cos_sin.data_ptr() if folds else 0, 1 if uneven and decode else 0, pieces, piece_stride,
+            1 if self.force_generic else 0, self.stream)
         if rc != 0:
             # a launch that did not run whole may have left tickets behind, and a later launch that found
             # them non-zero would never recognise its last workgroup: clear them (a fill kernel) before
