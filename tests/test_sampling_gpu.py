@@ -77,6 +77,11 @@ def test_reference_vectors(kn):
     wide[2] = -1.0
     tok, *_ = run(kn, wide, SamplingParams())
     assert tok == [500, 128255, 0]
+    wider = torch.zeros((2, 262147))  # beyond every vocabulary that a kernel here is tuned for
+    wider[0, [262146, 131072]] = 2.0
+    wider[1, 262146] = 1.0
+    tok, *_ = run(kn, wider, SamplingParams())
+    assert tok == [131072, 262146]
     for seed in range(30):
         h = [[0]] 
         tok, kept, *_ = run(kn, torch.tensor([[2.0, 10.0, 5.0, 1.0]]), SamplingParams(temperature=1.0, top_k=1, seed=seed), history=h)
@@ -89,7 +94,7 @@ def test_reference_vectors(kn):
     assert tok == [0] and lg[0].tolist() == [0.800000011920929, 0.5, 0.800000011920929]
 
 
-@pytest.mark.parametrize("vocab", [331, 4096, 128256])
+@pytest.mark.parametrize("vocab", [331, 4096, 128256, 262147])
 @pytest.mark.parametrize("temperature,top_k,top_p", [(0.8, 0, 1.0), (1.0, 40, 1.0), (0.7, 0, 0.9), (0.7, 40, 0.95),
                                                     (1.3, 5, 0.5), (0.5, 1000, 0.999)])
 def test_kept_set_and_draw_follow_the_plain_sampler(kn, vocab, temperature, top_k, top_p):
@@ -107,7 +112,7 @@ def test_kept_set_and_draw_follow_the_plain_sampler(kn, vocab, temperature, top_
     assert state.rng_ctr.cpu().tolist()[:6] == [1, 0, 1, 1, 0, 1]  # each sampled sequence moved on by one draw
 
 
-@pytest.mark.parametrize("vocab", [8192, 50021, 128256, 131072])
+@pytest.mark.parametrize("vocab", [8192, 50021, 128256, 131072, 200003])
 @pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, 40, 1.0), (0.7, 40, 0.95), (1.3, 5, 0.5), (0.8, 1, 1.0),
                                                     (0.5, 64, 0.999), (2.0, 17, 0.3)])
 def test_a_small_top_k_worked_on_in_parts_gives_what_the_one_block_kernel_and_the_plain_sampler_give(
