@@ -8,15 +8,19 @@
 // out[r, :] = float(table[token[r], :])   (row copy, internal/device/kernels.metal:465-467)
 // A token that is no row of the table (a replayed step can be handed the sampler's "no token" before the
 // host has seen it) gives a row of zeros: nothing outside the table is read.
+// A packed table (the layout of lq_pack_weight, for a table that is also the head's weight) keeps 8 rows'
+// slabs of 64 elements side by side: element k of row n lies at (n / 8) 8 D + (k / 64) 512 + (n % 8) 64 + k % 64.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
-                             float* __restrict__ out, int D, int vocab) {
+                             float* __restrict__ out, int D, int vocab, int packed) {
   const int r = blockIdx.x;
   const long long tok = tokens[r];
   const bool known = tok >= 0 && tok < vocab;
-  const T* src = table + (known ? tok : 0) * (long long)D;
+  const long long row = known ? tok : 0;
+  const T* src = packed ? table + (row >> 3) * 8 * (long long)D + (row & 7) * 64 : table + row * (long long)D;
   float* dst = out + (long long)r * D;
-  for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = known ? to_f32(src[j]) : 0.0f;
+  for (int j = threadIdx.x; j < D; j += blockDim.x)
+    dst[j] = known ? to_f32(src[packed ? ((j >> 6) << 9) + (j & 63) : j]) : 0.0f;
 }
 
 // A bfloat16 row of a width that is a multiple of 8, 16 bytes a lane and load: all of a thread's loads are on
@@ -27,18 +31,21 @@ typedef float embed_f32x4 __attribute__((ext_vector_type(4)));
 template <int PER_THREAD>
 __global__ __launch_bounds__(256) void embed_bf16_vec_kernel(const bf16_t* __restrict__ table,
                                                              const int* __restrict__ tokens, float* __restrict__ out,
-                                                             int D, int vocab) {
+                                                             int D, int vocab, int packed) {
   const int r = blockIdx.x;
   const long long tok = tokens[r];
   const bool known = tok >= 0 && tok < vocab;
-  const embed_u32x4* src = (const embed_u32x4*)(table + (known ? tok : 0) * (long long)D);
+  const long long row = known ? tok : 0;
+  // (chunk c of 8 elements: packed, 8 chunks of a row every 64 chunks)
+  const embed_u32x4* src = (const embed_u32x4*)(packed ? table + (row >> 3) * 8 * (long long)D + (row & 7) * 64
+                                                       : table + row * (long long)D);
   embed_f32x4* dst = (embed_f32x4*)(out + (long long)r * D);
   const int chunks = D / 8;
   embed_u32x4 v[PER_THREAD];
 #pragma unroll
   for (int i = 0; i < PER_THREAD; ++i) {
     const int c = threadIdx.x + i * 256;
-    v[i] = (c < chunks && known) ? src[c] : (embed_u32x4){0u, 0u, 0u, 0u};
+    v[i] = (c < chunks && known) ? src[packed ? ((c >> 3) << 6) + (c & 7) : c] : (embed_u32x4){0u, 0u, 0u, 0u};
   }
 #pragma unroll
   for (int i = 0; i < PER_THREAD; ++i) {
@@ -53,27 +60,55 @@ __global__ __launch_bounds__(256) void embed_bf16_vec_kernel(const bf16_t* __res
 }
 
 extern "C" int lq_embed(const void* table, int table_dtype, const int* tokens, float* out, int rows,
-                        int D, int vocab, hipStream_t stream) {
+                        int D, int vocab, int packed, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && D > 0 && vocab > 0, "embed: rows %d, width %d and table rows %d must be positive", rows, D, vocab);
+  LQ_REQUIRE(!packed || (D % 64 == 0 && vocab % 8 == 0), "embed: a packed table has rows in eights and a width in 64s");
   const int threads = D >= 1024 ? 256 : 64;
   if (table_dtype == LQ_BF16 && D % 8 == 0 && D >= 2048 && D <= 8 * 256 * 8 && (uintptr_t)table % 16 == 0 &&
       (uintptr_t)out % 16 == 0) {
     if (D <= 8 * 256 * 2)
-      embed_bf16_vec_kernel<2><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab);
+      embed_bf16_vec_kernel<2><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed);
     else if (D <= 8 * 256 * 4)
-      embed_bf16_vec_kernel<4><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab);
+      embed_bf16_vec_kernel<4><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed);
     else
-      embed_bf16_vec_kernel<8><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab);
+      embed_bf16_vec_kernel<8><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed);
     LQ_CHECK_LAUNCH("embed");
     return 0;
   }
   if (table_dtype == LQ_F32)
-    embed_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, tokens, out, D, vocab);
+    embed_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, tokens, out, D, vocab, packed);
   else if (table_dtype == LQ_BF16)
-    embed_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab);
+    embed_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed);
   else
     LQ_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
   LQ_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------- packed weights
+// dst = src [N, K] with 8 rows' slabs of 64 k side by side: element k of row n at
+// (n / 8) 8 K + (k / 64) 512 + (n % 8) 64 + k % 64.  A kernel that fetches a slab of 64 k of 8 (or 128) rows
+// then reads one run of 1 KiB (16 KiB) instead of 128 bytes from each of 8 (128) places a row apart, and the
+// next slab is the next KiB: what the memory gives whole pages for.  N % 8 == 0, K % 64 == 0; 16 bytes a thread.
+__global__ __launch_bounds__(256) void pack_weight_kernel(const embed_u32x4* __restrict__ src,
+                                                          embed_u32x4* __restrict__ dst, long long chunks, int K) {
+  const long long c = (long long)blockIdx.x * 256 + threadIdx.x;  // chunk of 8 elements, in the order of dst
+  if (c >= chunks) return;
+  const long long per8 = (long long)K;       // chunks in 8 rows: 8 K / 8
+  const long long group = c / per8, in = c - group * per8;
+  const int slab = (int)(in >> 6), row = (int)(in >> 3) & 7, part = (int)in & 7;
+  dst[c] = src[((group * 8 + row) * (long long)K + slab * 64 + part * 8) >> 3];
+}
+
+extern "C" int lq_pack_weight(const void* src, void* dst, int N, int K, hipStream_t stream) {
+  LQ_REQUIRE(src && dst && src != dst, "pack_weight: two different buffers");
+  LQ_REQUIRE(N > 0 && K > 0 && N % 8 == 0 && K % 64 == 0, "pack_weight: %d rows in eights, %d columns in 64s", N, K);
+  LQ_REQUIRE((uintptr_t)src % 16 == 0 && (uintptr_t)dst % 16 == 0, "pack_weight: 16-byte aligned buffers");
+  const long long chunks = (long long)N * K / 8;
+  LQ_REQUIRE((chunks + 255) / 256 < (1ll << 31), "pack_weight: too large");
+  pack_weight_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, stream>>>((const embed_u32x4*)src, (embed_u32x4*)dst,
+                                                                           chunks, K);
+  LQ_CHECK_LAUNCH("pack_weight");
   return 0;
 }
 

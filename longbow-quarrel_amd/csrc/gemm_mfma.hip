@@ -312,7 +312,7 @@ struct PipeShape {
 template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO, bool ALTERNATE = false>
 __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw, TO* __restrict__ C, int ldc, int M,
-    int N, int K, int tiles_m, int tiles_n, int k_share, long long split_stride) {
+    int N, int K, int tiles_m, int tiles_n, int k_share, long long split_stride, int packed) {
   using S = PipeShape<GM, GN, WM, WN, BK, STAGES>;
   extern __shared__ __attribute__((aligned(1024))) unsigned char plds[];
 
@@ -343,16 +343,21 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
   // where this lane's 16 bytes of each transfer come from: transfer x = NW j + wave fills the stage's
   // chunks [64 x, 64 x + 64); chunk p is stage row p / CPR (A rows first), position p % CPR.  The address
   // is a wave-uniform origin (the operand's tile at this block's first k) plus a 32-bit lane offset.
+  // (a packed W keeps 8 rows' 64-k slabs side by side: slab s of rows 8 i .. 8 i + 7 is the KiB at
+  // element 8 i ldw + 512 s, a row's 64 k every 128 bytes in it; n0 and k_begin are multiples of 8 and 64)
+  const int w_kmul = packed ? 16 : 2;  // bytes that one k moves a slab's address on
   const char* a_origin = (const char*)(A + (long long)m0 * lda + k_begin);
-  const char* w_origin = (const char*)(W + (long long)n0 * ldw + k_begin);
+  const char* w_origin = (const char*)(W + (long long)n0 * ldw) + (long long)k_begin * w_kmul;
   unsigned off[S::DMA];
   int dst[S::DMA];
 #pragma unroll
   for (int j = 0; j < S::DMA; ++j) {
     const int x = min(j * S::NW + wave, S::TRANSFERS - 1);
     const int p = x * 64 + lane, row = p / S::CPR, c = (p % S::CPR) ^ S::swizzle(row);
+    const unsigned wr = (unsigned)(min(n0 + row - S::BM, N - 1) - n0);
     off[j] = row < S::BM ? (unsigned)(min(m0 + row, M - 1) - m0) * (unsigned)lda * 2u + c * 16
-                         : (unsigned)(min(n0 + row - S::BM, N - 1) - n0) * (unsigned)ldw * 2u + c * 16;
+             : packed    ? (wr >> 3) * (unsigned)ldw * 16u + (wr & 7) * 128u + c * 16
+                         : wr * (unsigned)ldw * 2u + c * 16;
     dst[j] = x * 1024;
   }
   auto dma = [&](int stage, int k0) {
@@ -360,7 +365,7 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
 #pragma unroll
     for (int j = 0; j < S::DMA; ++j) {
       // a scalar base and a 32-bit lane offset: one address register a transfer
-      const char* origin = uniform_ptr((j < S::A_ROUNDS ? a_origin : w_origin) + (long long)k0 * 2);
+      const char* origin = uniform_ptr(j < S::A_ROUNDS ? a_origin + (long long)k0 * 2 : w_origin + (long long)k0 * w_kmul);
       __builtin_amdgcn_global_load_lds(LQ_GLOBAL_PTR(origin + off[j]), LQ_LDS_PTR(base + dst[j]), 16, 0, 0);
     }
   };
@@ -459,8 +464,12 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
     const int lrow = lane / S::CPR;
     const int lchunk = ((lane % S::CPR) ^ S::swizzle(w4 * S::ROWS_PER_DMA + lrow)) * 16;
     const int ld = group == 0 ? ldw : lda;
-    const int t_voff = (w4 * S::ROWS_PER_DMA + lrow) * ld * 2 + lchunk;  // this lane in the wave's transfer 0
-    const int t_step = 4 * S::ROWS_PER_DMA * ld * 2;                      // to the wave's next transfer
+    static_assert(!ALTERNATE || S::ROWS_PER_DMA == 8, "a transfer is the 8 rows that a packed W keeps together");
+    const bool w_packed = group == 0 && packed;
+    // this lane in the wave's transfer 0, and the way to the wave's next transfer
+    const int t_voff = w_packed ? w4 * ld * 16 + lrow * 128 + lchunk : (w4 * S::ROWS_PER_DMA + lrow) * ld * 2 + lchunk;
+    const int t_step = 4 * S::ROWS_PER_DMA * ld * 2;
+    const int t_kmul = w_packed ? 16 : 2;
     const __amdgpu_buffer_rsrc_t t_rsrc =
         group == 0 ? __builtin_amdgcn_make_buffer_rsrc((void*)w_origin, 0, min(N - n0, S::BN) * ldw * 2, 0x00020000)
                    : __builtin_amdgcn_make_buffer_rsrc((void*)a_origin, 0, min(M - m0, S::BM) * lda * 2, 0x00020000);
@@ -469,7 +478,7 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
       int v = t_voff;
       asm volatile("" : "+v"(v));  // added up anew every time: kept across the loop it would cost a register a transfer
       __builtin_amdgcn_raw_ptr_buffer_load_lds(t_rsrc, LQ_LDS_PTR(plds + stage * S::STAGE_BYTES + t_dst + j * 4096), 16,
-                                               v + j * t_step, k0 * 2, 0, 0);
+                                               v + j * t_step, k0 * t_kmul, 0, 0);
     };
     for (int q = 0; q < 2 && q < slabs; ++q)
 #pragma unroll
@@ -559,8 +568,9 @@ __global__ __launch_bounds__(GM * GN * 64, 2) void gemm_bf16_pipelined_kernel(
 
 template <int GM, int GN, int WM, int WN, int BK, int STAGES, int EPI, typename TO, bool ALTERNATE = false>
 int launch_pipelined(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
-                     int splits, long long split_stride, hipStream_t stream) {
+                     int splits, long long split_stride, hipStream_t stream, int packed = 0) {
   using S = PipeShape<GM, GN, WM, WN, BK, STAGES>;
+  LQ_REQUIRE(!packed || (BK == 64 && N % 8 == 0), "linear: a packed weight needs slabs of 64 k and rows in eights");
   const int tiles_m = lq_ceil_div(M, S::BM), tiles_n = lq_ceil_div(N, S::BN);
   auto kernel = gemm_bf16_pipelined_kernel<GM, GN, WM, WN, BK, STAGES, EPI, TO, ALTERNATE>;
   static bool configured = false;
@@ -581,7 +591,8 @@ int launch_pipelined(const void* A, const void* W, void* C, int M, int N, int K,
   LQ_REQUIRE((long long)lda * 2 * S::BM < (1ll << 31) && (long long)ldw * 2 * S::BN < (1ll << 31),
              "linear: rows too far apart for the tile's 32-bit offsets");
   kernel<<<dim3((int)blocks, splits), S::NW * 64, S::LDS_BYTES, stream>>>(
-      (const bf16_t*)A, lda, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, tiles_m, tiles_n, K / splits, split_stride);
+      (const bf16_t*)A, lda, (const bf16_t*)W, ldw, (TO*)C, ldc, M, N, K, tiles_m, tiles_n, K / splits, split_stride,
+      packed);
   LQ_CHECK_LAUNCH("linear(mfma pipelined)");
   return 0;
 }
@@ -702,7 +713,7 @@ struct ResidualOut {
   int ld_scaled;
 };
 
-template <int KW, int MT, int EPI, typename TO, bool SCALED>
+template <int KW, int MT, int EPI, typename TO, bool SCALED, bool PACKED>
 __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16_t* __restrict__ X, int ldx,
                                                                       const bf16_t* __restrict__ W, int ldw,
                                                                       TO* __restrict__ C, int ldc, int M, int N,
@@ -765,12 +776,15 @@ __global__ __launch_bounds__(KW * 64) void gemm_bf16_skinny_v3_kernel(const bf16
     for (int t = 0; t < V3_MAXT; ++t) {
       if (t < ntiles) {
         const int nrow = min(col_begin + t * 16 + c16, col_end - 1);
-        const bf16_t* wp = W + (long long)nrow * ldw;
+        // (packed: 8 rows' slabs of 64 k side by side; a wave's slice starts at a multiple of 64, so step s is
+        // a constant number of bytes from the slice's first slab, as in a dense row)
+        const bf16_t* wp = PACKED ? W + (long long)(nrow >> 3) * 8 * ldw + (nrow & 7) * 64 + ((kb >> 6) << 9) + g * 8
+                                  : W + (long long)nrow * ldw + kb + g * 8;
         u32x4 wv[KB];
 #pragma unroll
         for (int s = 0; s < KB; ++s) {
           const int k = kb + s * 32 + g * 8;
-          wv[s] = (k < k_stop) ? *(const u32x4*)(wp + k) : zero;
+          wv[s] = (k < k_stop) ? *(const u32x4*)(wp + (PACKED ? (s >> 1) * 512 + (s & 1) * 32 : s * 32)) : zero;
         }
 #pragma unroll
         for (int s = 0; s < KB; ++s)
@@ -907,16 +921,34 @@ inline void v3_runs(int N, int cus, int unit, int& cols, int& grid) {
   grid = lq_ceil_div(N, cols);
 }
 
+template <int KW, int MT, int EPI, typename TO, bool SCALED, bool PACKED>
+int launch_skinny_v3_as(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc, int splits,
+                        long long split_stride, hipStream_t stream, RowScale scale, ResidualOut res, int cols, int grid,
+                        int ks_per_wave);
+
 template <int MT, int EPI, typename TO, bool SCALED = false>
 int launch_skinny_v3(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc,
-                     int splits, long long split_stride, hipStream_t stream, RowScale scale = RowScale(),
-                     ResidualOut res = ResidualOut()) {
+                     int splits, long long split_stride, hipStream_t stream, int packed = 0,
+                     RowScale scale = RowScale(), ResidualOut res = ResidualOut()) {
   constexpr int KW = v3_kw(MT);
+  LQ_REQUIRE(!packed || (K % 64 == 0 && N % 8 == 0), "linear: a packed weight has K in 64s and rows in eights");
   int cols, grid;
   v3_runs(N, lq_compute_units() / splits, EPI == EPI_SWIGLU ? 16 : 8, cols, grid);
   const int ksteps = lq_ceil_div(K, 32);
-  const int ks_per_wave = lq_ceil_div(ksteps, KW * splits);
-  auto kernel = gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO, SCALED>;
+  // an even number of 32-k steps a wave: its slice starts at a multiple of 64, where a packed weight's slabs do
+  const int ks_per_wave = (lq_ceil_div(ksteps, KW * splits) + 1) / 2 * 2;
+  if (packed)
+    return launch_skinny_v3_as<KW, MT, EPI, TO, SCALED, true>(X, W, C, M, N, K, ldx, ldw, ldc, splits, split_stride, stream,
+                                                              scale, res, cols, grid, ks_per_wave);
+  return launch_skinny_v3_as<KW, MT, EPI, TO, SCALED, false>(X, W, C, M, N, K, ldx, ldw, ldc, splits, split_stride, stream,
+                                                             scale, res, cols, grid, ks_per_wave);
+}
+
+template <int KW, int MT, int EPI, typename TO, bool SCALED, bool PACKED>
+int launch_skinny_v3_as(const void* X, const void* W, void* C, int M, int N, int K, int ldx, int ldw, int ldc, int splits,
+                        long long split_stride, hipStream_t stream, RowScale scale, ResidualOut res, int cols, int grid,
+                        int ks_per_wave) {
+  auto kernel = gemm_bf16_skinny_v3_kernel<KW, MT, EPI, TO, SCALED, PACKED>;
   // one row tile: a KiB of LDS for every column tile and wave of a block
   const int lds = MT == 1 ? lq_ceil_div(cols, 16) * KW * 1024 : 0;
   static bool configured = false;
@@ -945,6 +977,12 @@ int pick_skinny(const void* x, const void* w, void* out, int M, int N, int K, in
   if (tiles * 8 >= 2048 || chunks < 16 || MT > 2)
     return launch_skinny<8, MT, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   return launch_skinny<16, MT, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
+}
+
+// A weight may be kept packed (8 rows' slabs of 64 k side by side, see lq_gemm_pack_layout) if every product
+// with it runs in the pipelined kernel with slabs of 64 k or in the balanced kernel: wide, K in 64s.
+inline bool gemm_packable(int N, int K) {
+  return N >= 8 * lq_compute_units() && N % 8 == 0 && K >= 512 && K % 64 == 0;
 }
 
 // The large pipelined tile pays once its tiles (times the shares of K) fill three quarters of the chip.
@@ -998,29 +1036,29 @@ int mid_splits(int M, int N, int K) {
 
 template <int EPI, typename TO>
 int launch_mid(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc, int splits,
-               long long split_stride, hipStream_t stream) {
+               long long split_stride, hipStream_t stream, int packed) {
   // whole and with few columns: 64- or 32-column tiles (no epilogue pairs columns across them)
   if constexpr (EPI == EPI_NONE) {
     const int want = 3 * lq_compute_units() / 4;
     if (splits == 1 && lq_ceil_div(N, 64) < want) {
-      if (M <= 64) return launch_pipelined<2, 1, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
-      if (M <= 128) return launch_pipelined<4, 1, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
-      return launch_pipelined<8, 1, 1, 1, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      if (M <= 64) return launch_pipelined<2, 1, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
+      if (M <= 128) return launch_pipelined<4, 1, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
+      return launch_pipelined<8, 1, 1, 1, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
     }
     if (splits == 1 && lq_ceil_div(N, 128) < want) {
-      if (M <= 64) return launch_pipelined<2, 2, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
-      if (M <= 128) return launch_pipelined<2, 2, 2, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
-      return launch_pipelined<4, 2, 2, 1, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      if (M <= 64) return launch_pipelined<2, 2, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
+      if (M <= 128) return launch_pipelined<2, 2, 2, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
+      return launch_pipelined<4, 2, 2, 1, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
     }
   }
   if constexpr (EPI == EPI_NONE)
     if (splits > 1 && mid_narrow(M, N, K))
-      return launch_pipelined<2, 2, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+      return launch_pipelined<2, 2, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
   if (M <= 64)
-    return launch_pipelined<2, 4, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+    return launch_pipelined<2, 4, 1, 1, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
   if (M <= 128)
-    return launch_pipelined<4, 2, 1, 2, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
-  return launch_pipelined<4, 2, 2, 2, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+    return launch_pipelined<4, 2, 1, 2, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
+  return launch_pipelined<4, 2, 2, 2, 64, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
 }
 
 int mfma_splits(int M, int N, int K) {
@@ -1030,32 +1068,35 @@ int mfma_splits(int M, int N, int K) {
 
 template <int EPI, typename TO>
 int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int lda, int ldw, int ldc,
-             int splits, long long split_stride, hipStream_t stream) {
+             int splits, long long split_stride, hipStream_t stream, int packed) {
+  // a packed weight is wide and has K in 64s (gemm_packable): every way below that it can take ends in the
+  // pipelined kernel with slabs of 64 k or in the balanced one
+  LQ_REQUIRE(!packed || gemm_packable(N, K), "linear: a %d x %d weight cannot be packed", N, K);
   if (splits > 1) {
     if (EPI != EPI_NONE || splits != mfma_splits(M, N, K)) {
       lq_set_error("linear: %d shares of K are not what this product takes (%d)", splits, mfma_splits(M, N, K));
       return -1;
     }
   }
-  if (mid_rows(M, N, K)) return launch_mid<EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+  if (mid_rows(M, N, K)) return launch_mid<EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
   if (splits > 1) {
-    if (M <= 32) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
-    if (M <= 64) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+    if (M <= 32) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
+    if (M <= 64) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
     return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride,
-                                                              stream);
+                                                              stream, packed);
   }
   // wide enough to give every compute unit a run of columns: the balanced kernel; else the simple one
   const bool wide = N >= 8 * lq_compute_units() && K >= 512;
   if (M <= 16) {
-    if (wide) return launch_skinny_v3<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    if (wide) return launch_skinny_v3<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
     return pick_skinny<1, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
   if (M <= 32) {
-    if (wide) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    if (wide) return launch_skinny_v3<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
     return pick_skinny<2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
   if (M <= 64) {
-    if (wide) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    if (wide) return launch_skinny_v3<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
     return pick_skinny<4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   }
   // the largest tile that still fills the chip: 256 rows by 256, 224 or 192 columns (8 waves), 128 x 256
@@ -1079,22 +1120,22 @@ int dispatch(const void* x, const void* w, void* out, int M, int N, int K, int l
       if (N % 256 == 0 && tm * tn > cus && 4 * rest >= cus && rest % tm == 0 && 2 * rest <= cus + cus / 8) {
         const int n1 = (tn - rest / tm) * 256, n2 = N - n1;
         const int col2 = EPI == EPI_SWIGLU ? n1 / 2 : n1;  // where the second launch's columns start in out
-        int rc = launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, n1, K, lda, ldw, ldc, 1, 0, stream);
+        int rc = launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, n1, K, lda, ldw, ldc, 1, 0, stream, packed);
         if (rc != 0) return rc;
         return launch_pipelined<4, 2, 2, 2, 64, 2, EPI, TO, true>(x, (const bf16_t*)w + (long long)n1 * ldw,
-                                                                  (TO*)out + col2, M, n2, K, lda, ldw, ldc, 1, 0, stream);
+                                                                  (TO*)out + col2, M, n2, K, lda, ldw, ldc, 1, 0, stream, packed);
       }
-      return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      return launch_pipelined<4, 2, 2, 4, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
     }
     if (c224 <= c192)
-      return launch_pipelined<8, 1, 1, 7, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
-    return launch_pipelined<4, 2, 2, 3, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+      return launch_pipelined<8, 1, 1, 7, 64, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
+    return launch_pipelined<4, 2, 2, 3, 64, 2, EPI, TO, true>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
   }
-  if (K % 32 == 0 && t128 >= lq_compute_units())
-    return launch_pipelined<2, 2, 2, 4, 32, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+  if (!packed && K % 32 == 0 && t128 >= lq_compute_units())
+    return launch_pipelined<2, 2, 2, 4, 32, 3, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
   // few tiles even of 128 x 256 (some hundred rows of a narrow matrix): 128 x 128 tiles, four stages deep
   if (K % 64 == 0 && K >= 512)
-    return launch_pipelined<4, 2, 1, 2, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    return launch_pipelined<4, 2, 1, 2, 64, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
   if (t128 >= 2 * lq_compute_units()) return launch_tiled<2, 4, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
   return launch_tiled<2, 2, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
 }
@@ -1116,17 +1157,18 @@ int lq_gemm_fused_parts(int M, int N, int K) {
 }
 
 int lq_gemm_residual(const void* act, const void* w, float* x, float* sq_out, const float* gain, void* scaled,
-                     int ld_scaled, int M, int N, int K, int lda, int ldw, int ldx, hipStream_t stream) {
+                     int ld_scaled, int M, int N, int K, int lda, int ldw, int ldx, int packed, hipStream_t stream) {
   ResidualOut res;
   res.sq_out = sq_out;
   res.gain = gain;
   res.scaled = (bf16_t*)scaled;
   res.ld_scaled = ld_scaled;
-  return launch_skinny_v3<1, EPI_RESIDUAL, float>(act, w, x, M, N, K, lda, ldw, ldx, 1, 0, stream, RowScale(), res);
+  return launch_skinny_v3<1, EPI_RESIDUAL, float>(act, w, x, M, N, K, lda, ldw, ldx, 1, 0, stream, packed, RowScale(), res);
 }
 
 int lq_gemm_scaled(const void* h, int ldh, const float* sq_parts, int n_parts, int width, float eps, const void* w,
-                   void* out, int out_dtype, int M, int N, int K, int ldw, int ldc, int swiglu, hipStream_t stream) {
+                   void* out, int out_dtype, int M, int N, int K, int ldw, int ldc, int swiglu, int packed,
+                   hipStream_t stream) {
   RowScale sc;
   sc.sq_parts = sq_parts;
   sc.n_parts = n_parts;
@@ -1134,14 +1176,14 @@ int lq_gemm_scaled(const void* h, int ldh, const float* sq_parts, int n_parts, i
   sc.eps = eps;
   if (swiglu) {
     if (out_dtype == LQ_BF16)
-      return launch_skinny_v3<1, EPI_SWIGLU, bf16_t, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, sc);
+      return launch_skinny_v3<1, EPI_SWIGLU, bf16_t, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, packed, sc);
     if (out_dtype == LQ_F32)
-      return launch_skinny_v3<1, EPI_SWIGLU, float, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, sc);
+      return launch_skinny_v3<1, EPI_SWIGLU, float, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, packed, sc);
   } else {
     if (out_dtype == LQ_BF16)
-      return launch_skinny_v3<1, EPI_NONE, bf16_t, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, sc);
+      return launch_skinny_v3<1, EPI_NONE, bf16_t, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, packed, sc);
     if (out_dtype == LQ_F32)
-      return launch_skinny_v3<1, EPI_NONE, float, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, sc);
+      return launch_skinny_v3<1, EPI_NONE, float, true>(h, w, out, M, N, K, ldh, ldw, ldc, 1, 0, stream, packed, sc);
   }
   lq_set_error("linear: unknown output dtype %d", out_dtype);
   return -1;
@@ -1153,20 +1195,22 @@ bool lq_gemm_mfma_accepts(const void* x, const void* w, int in_dtype, int K, int
          ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
 }
 
+bool lq_gemm_packable(int N, int K) { return gemm_packable(N, K); }
+
 int lq_gemm_mfma(const void* x, const void* w, void* out, int out_dtype, int M, int N, int K, int lda,
-                 int ldw, int ldc, int epilogue, int splits, long long split_stride, hipStream_t stream) {
+                 int ldw, int ldc, int epilogue, int splits, long long split_stride, int packed, hipStream_t stream) {
   if (epilogue == EPI_NONE) {
     if (out_dtype == LQ_F32)
-      return dispatch<EPI_NONE, float>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+      return dispatch<EPI_NONE, float>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
     if (out_dtype == LQ_BF16)
-      return dispatch<EPI_NONE, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream);
+      return dispatch<EPI_NONE, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, splits, split_stride, stream, packed);
   } else if (epilogue == EPI_SWIGLU) {
     if (N % 16 != 0) {
       lq_set_error("linear+swiglu: %d interleaved rows are not a multiple of 16", N);
       return -1;
     }
-    if (out_dtype == LQ_F32) return dispatch<EPI_SWIGLU, float>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
-    if (out_dtype == LQ_BF16) return dispatch<EPI_SWIGLU, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream);
+    if (out_dtype == LQ_F32) return dispatch<EPI_SWIGLU, float>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
+    if (out_dtype == LQ_BF16) return dispatch<EPI_SWIGLU, bf16_t>(x, w, out, M, N, K, lda, ldw, ldc, 1, 0, stream, packed);
   }
   lq_set_error("linear: unknown out dtype %d or epilogue %d", out_dtype, epilogue);
   return -1;

@@ -15,7 +15,7 @@ void lq_set_error(const char* fmt, ...) {
 
 extern "C" const char* lq_last_error() { return g_error; }
 
-extern "C" int lq_abi_version() { return 4; }
+extern "C" int lq_abi_version() { return 5; }
 
 // Compute units of the current device (256 if the runtime will not say).
 int lq_compute_units() {

@@ -20,7 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
-ABI_VERSION = 4  # lq_abi_version() of the library these wrappers were written for
+ABI_VERSION = 5  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -55,8 +55,8 @@ def load_library() -> ctypes.CDLL:
     # save making a ctypes object for each of them: a call from Python is 5 us instead of 10, where the
     # launch itself is 3).
     vp, ci, cl, cf = c_void_p, c_int, c_longlong, c_float
-    lib.lq_linear.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cl, ci, vp]
-    lib.lq_linear_swiglu.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp]
+    lib.lq_linear.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cl, ci, ci, vp]
+    lib.lq_linear_swiglu.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]
     lib.lq_rmsnorm.argtypes = [vp, vp, ci, ci, cl, vp, cf, vp, ci, ci, ci, vp]
     lib.lq_attention.argtypes = [vp, ci, vp, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, vp, vp, ci, vp, vp, ci, cf, ci, ci, ci,
                                  vp, cl, vp, cl, vp, vp, ci, ci, vp, ci, ci, cl, ci, vp]
@@ -79,6 +79,44 @@ def _code(t: torch.Tensor) -> int:
         raise KernelLibraryError(f"unsupported tensor dtype {t.dtype}") from None
 
 
+class PackedWeight:
+    """A weight [N, K] whose memory is in the packed order of `HipKernels.pack_weight`: what the products and
+    the embedding take in a tensor's place.  It answers what they ask of a weight (shape, dtype, strides of the
+    matrix it stands for, the address) and is no tensor: nothing else can read it by mistake."""
+
+    packed = True
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int) -> None:
+        self.data, self.shape, self.dtype, self.device = data, torch.Size((rows, cols)), data.dtype, data.device
+        self.is_cuda = data.is_cuda
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+    def dim(self) -> int:
+        return 2
+
+    def stride(self, i: Optional[int] = None):
+        st = (self.shape[1], 1)
+        return st if i is None else st[i]
+
+    def is_contiguous(self) -> bool:
+        return True
+
+    def contiguous(self) -> "PackedWeight":
+        return self
+
+    def numel(self) -> int:
+        return self.data.numel()
+
+    def element_size(self) -> int:
+        return self.data.element_size()
+
+
+def _packed(w) -> int:
+    return 1 if getattr(w, "packed", False) else 0
+
+
 class HipKernels:
     name = "hip-gfx950"
 
@@ -88,6 +126,7 @@ class HipKernels:
             raise KernelLibraryError("no HIP device is visible; this library runs on a gfx950 GPU only")
         self._stream: Optional[int] = None
         self.force_generic = False  # route linear and attention to the size-agnostic kernels
+        self.pack_weights = True    # `pack_weight` packs what may be packed (False: it hands every weight back)
         # ticket counters of the decoding attention (one for each row and kv head of a launch); a launch
         # finds them zero and leaves them zero, so launches through one object must not overlap
         self._tickets: dict = {}  # device -> the counters
@@ -169,6 +208,22 @@ class HipKernels:
             raise KernelLibraryError(f"{what}: need a contiguous int32 tensor of at least {n} entries")
 
     # ------------------------------------------------------------------ kernels
+    def pack_weight(self, w: torch.Tensor):
+        """The weight [N, K] of a product as the products like to read it, made once when weights are bound:
+        a `PackedWeight` (8 rows' slabs of 64 k side by side, so that the slab of a tile of rows is one run of
+        memory instead of 128 bytes from every row) where every kernel that can meet a weight of this size reads
+        that order (bfloat16, wide, K in 64s), else w itself.  `linear`, `linear_swiglu`, `linear_residual`,
+        `linear_scaled` and `embed` take either."""
+        if not self.pack_weights or getattr(w, "packed", False) or w.dim() != 2 or w.dtype not in _DTYPE_CODE \
+                or not w.is_cuda or not w.is_contiguous():
+            return w
+        n, k = w.shape
+        if not self.lib.lq_weight_packable(c_int(_DTYPE_CODE[w.dtype]), c_int(n), c_int(k)):
+            return w
+        out = torch.empty_like(w)
+        self._check(self.lib.lq_pack_weight(_ptr(w), _ptr(out), c_int(n), c_int(k), self.stream))
+        return PackedWeight(out, n, k)
+
     def embed(self, table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
         """out[r, :] = float32(table[tokens[r], :]); zeros where tokens[r] is no row of the table"""
         self._dev(table, tokens, out)
@@ -179,7 +234,8 @@ class HipKernels:
         if table.dim() != 2 or table.shape[1] != width:
             raise KernelLibraryError(f"embed: table {tuple(table.shape)} does not match width {width}")
         self._check(self.lib.lq_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(out),
-                                      c_int(rows), c_int(width), c_int(table.shape[0]), self.stream))
+                                      c_int(rows), c_int(width), c_int(table.shape[0]), c_int(_packed(table)),
+                                      self.stream))
 
     @staticmethod
     def _pieces(delta: Optional[torch.Tensor], like: torch.Tensor, what: str):
@@ -258,7 +314,7 @@ class HipKernels:
         if x.dtype != w.dtype:
             raise KernelLibraryError(f"linear: x is {x.dtype} but w is {w.dtype}")
         rc = self.lib.lq_linear(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(x), _code(out), m, n, k, ldx, ldw,
-                                ldc, pieces, stride, 1 if self.force_generic else 0, self.stream)
+                                ldc, pieces, stride, 1 if self.force_generic else 0, _packed(w), self.stream)
         if rc:
             self._check(rc)
 
@@ -294,7 +350,8 @@ class HipKernels:
                                                 c_int(self._rows2d(scaled, "scaled") if scaled is not None else 0),
                                                 c_int(_code(act)), c_int(m), c_int(n), c_int(k),
                                                 c_int(self._rows2d(act, "act")), c_int(self._rows2d(w, "w")),
-                                                c_int(self._rows2d(x, "x")), c_int(sq_parts.shape[1]), self.stream))
+                                                c_int(self._rows2d(x, "x")), c_int(sq_parts.shape[1]),
+                                                c_int(_packed(w)), self.stream))
 
     def linear_scaled(self, h: torch.Tensor, sq_parts: torch.Tensor, eps: float, w: torch.Tensor,
                       out: torch.Tensor, swiglu: bool = False) -> None:
@@ -313,7 +370,7 @@ class HipKernels:
                                               c_int(sq_parts.shape[1]), c_float(eps), _ptr(w), _ptr(out),
                                               c_int(_code(w)), c_int(_code(out)), c_int(m), c_int(n), c_int(k),
                                               c_int(self._rows2d(w, "w")), c_int(self._rows2d(out, "out")),
-                                              c_int(1 if swiglu else 0), self.stream))
+                                              c_int(1 if swiglu else 0), c_int(_packed(w)), self.stream))
 
     @query
     def linear_swiglu_supported(self, dtype: torch.dtype, rows_out: int, k: int) -> bool:
@@ -333,7 +390,7 @@ class HipKernels:
             raise KernelLibraryError(
                 f"linear_swiglu: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
         rc = self.lib.lq_linear_swiglu(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(x), _code(out), m, n, k,
-                                       ldx, ldw, ldc, self.stream)
+                                       ldx, ldw, ldc, _packed(w), self.stream)
         if rc:
             self._check(rc)
 

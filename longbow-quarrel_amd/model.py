@@ -20,7 +20,8 @@ from typing import Dict, List, Mapping, Optional, Sequence
 import torch
 
 from .parts.base import (BLOCKS, EMBEDDINGS, LOGIT_STEPS, MATRIX, NORMS, Block, BuildEnv, Embedding, LogitsStep, Norm,
-                         NormedRows, PartSpec, RowStats, StepContext, TensorSpec, build_part, project, project_normed)
+                         NormedRows, PartSpec, RowStats, StepContext, TensorSpec, build_part, product_weight, project,
+                         project_normed)
 
 
 @dataclass(frozen=True)
@@ -94,12 +95,15 @@ class DecoderModel:
         for p in self.parts():
             p.bind(tensors, env)
         if s.head_name is not None and not s.tie_head:
-            self.head = tensors[s.head_name].contiguous()
+            self.head = product_weight(env, tensors[s.head_name])
         else:
             # the head is the embedding when the file has none: internal/engine/engine.go:1106-1116
             table = self.embedding.table
             if table is None or tuple(table.shape) != (s.vocab_size, s.width):
                 raise ValueError("the output head is tied to the embedding, which has no [vocab, width] table")
+            if getattr(self.embedding, "table_is_for_kernels", False):
+                # one copy for both: the embedding's kernel reads the product's form of the table too
+                table = self.embedding.table = product_weight(env, table)
             self.head = table
 
     # ---- what the cache has to hold -----------------------------------------------

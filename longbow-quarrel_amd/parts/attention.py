@@ -18,7 +18,8 @@ from typing import Dict, List, Mapping, Optional
 import torch
 
 from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mixer, PartSpec,
-                   NormedRows, StepContext, TensorSpec, build_part, project, project_into, project_normed)
+                   NormedRows, StepContext, TensorSpec, build_part, product_weight, project, project_into,
+                   project_normed)
 
 
 @MIXERS.register("gqa_attention")
@@ -57,8 +58,8 @@ class GQAttention(Mixer):
         q, k, v = (tensors[self.names[key]] for key in ("q", "k", "v"))
         if not (q.dtype == k.dtype == v.dtype):
             raise ValueError(f"{self.names['q']}: q, k and v projections are stored in different dtypes")
-        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
-        self.w_o = tensors[self.names["o"]].contiguous()
+        self.w_qkv = product_weight(env, torch.cat([q, k, v], dim=0))
+        self.w_o = product_weight(env, tensors[self.names["o"]])
         self.position.bind(tensors, env)
 
     def cache_need(self) -> KVNeed:

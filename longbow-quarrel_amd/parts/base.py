@@ -508,6 +508,15 @@ def project_delta(kn, ctx: StepContext, x: torch.Tensor, w: torch.Tensor) -> tor
     return out
 
 
+def product_weight(env: BuildEnv, w: torch.Tensor):
+    """A weight [N, K] as the kernels' products like to hold it, asked once when weights are bound: what
+    `kernels.pack_weight` makes of it (something that `linear` and its siblings take in a tensor's place and that
+    still answers `.shape` and `.dtype`), or the dense tensor where the kernel object has no such method."""
+    w = w.contiguous()
+    pack = getattr(env.kernels, "pack_weight", None)
+    return pack(w) if pack is not None else w
+
+
 def project(kn, ctx: StepContext, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     """out = x . w^T.  A weight stored in 32-bit is used in 32-bit: bfloat16
     activations are widened for it rather than the weight narrowed."""

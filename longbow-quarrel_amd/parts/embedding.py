@@ -13,6 +13,9 @@ from .base import EMBEDDINGS, MATRIX, BuildEnv, Embedding, StepContext, TensorSp
 @EMBEDDINGS.register("token_table")
 class TokenTable(Embedding):
     graph_safe = True
+    # `table` is only ever handed to `kernels.embed`: a model whose head is this table may put the product's
+    # form of it (`parts.base.product_weight`) in its place
+    table_is_for_kernels = True
 
     def __init__(self, name: str, vocab_size: int, width: int) -> None:
         self.name, self.vocab_size, self.width = name, int(vocab_size), int(width)

@@ -8,8 +8,8 @@ from typing import Dict, List, Mapping, Optional
 
 import torch
 
-from .base import (FEED_FORWARDS, BuildEnv, FeedForward, NormedRows, StepContext, TensorSpec, project, project_into,
-                   project_normed)
+from .base import (FEED_FORWARDS, BuildEnv, FeedForward, NormedRows, StepContext, TensorSpec, product_weight, project,
+                   project_into, project_normed)
 
 
 @FEED_FORWARDS.register("swiglu")
@@ -42,10 +42,10 @@ class SwiGLU(FeedForward):
             getattr(kn, "linear_swiglu_supported", lambda *a: False)(gate.dtype, 2 * self.inner, self.width)
         if self.fused:
             # gate and up rows interleaved so that the product's epilogue can apply silu(g) * u itself
-            self.w_gate_up = kn.interleave_gate_up(gate, up)
+            self.w_gate_up = product_weight(env, kn.interleave_gate_up(gate, up))
         else:
-            self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
-        self.w_down = tensors[self.names["down"]].contiguous()
+            self.w_gate_up = product_weight(env, torch.cat([gate, up], dim=0))
+        self.w_down = product_weight(env, tensors[self.names["down"]])
 
     takes_normed_rows = True
     takes_residual_sink = True

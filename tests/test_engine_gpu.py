@@ -385,6 +385,41 @@ def test_decoding_with_add_and_norm_folded_into_the_projections(tmp_path_factory
     assert g1.tokens == g2.tokens
 
 
+def test_packed_weights_and_a_packed_tied_table_give_the_bits_of_dense_ones(tmp_path_factory):
+    """Wide weights are held packed (8 rows' slabs of 64 k side by side), the table of a tied head too, which the
+    embedding then reads in that order: the same logits, bit for bit, as an engine whose kernel object packs nothing,
+    for prompts of every kind of product (a few rows, 33 to 256, more) and for decoding steps."""
+    from longbow_quarrel_amd.kernels.hip import HipKernels
+
+    cfg = dict(WIDE, intermediate_size=2304, vocab_size=2056, tie_word_embeddings=True, num_hidden_layers=2)
+    folder = write_folder(tmp_path_factory.mktemp("packed"), cfg, seed=5, std=0.03)
+    engines = []
+    for pack in (True, False):
+        kn = HipKernels()
+        kn.pack_weights = pack
+        engines.append(lq.load_engine(folder, dtype="bfloat16", max_tokens=2048, kernels=kn))
+    packed, dense = engines
+    mixer, ff = packed.model.blocks[0].mixer, packed.model.blocks[0].ffn
+    for w in (mixer.w_qkv, mixer.w_o, ff.w_gate_up, ff.w_down, packed.model.head, packed.model.embedding.table):
+        assert getattr(w, "packed", False)
+    assert packed.model.head is packed.model.embedding.table
+    assert not any(getattr(w, "packed", False) for w in (dense.model.head, dense.model.blocks[0].mixer.w_qkv))
+    c, tensors = read_folder(folder)
+    ref = plain.PlainLlama(c, tensors)
+    prompt = random_tokens(400, cfg["vocab_size"], 77)
+    for n in (3, 16, 40, 130, 400):
+        outs = []
+        for eng in engines:
+            s = eng.new_sequence()
+            first = eng.step([StepEntry(s, prompt[:n], range(n))])
+            nxt = [eng.step([StepEntry(s, [prompt[n + i]], [0])]) for i in range(3)] if n < 400 else []
+            eng.release(s)
+            outs.append(torch.cat([first] + nxt))
+        assert torch.equal(outs[0], outs[1]), n
+        if n == 130:
+            assert rel_err(outs[0][:n], ref.forward(prompt[:n], plain.round_bf16)) < TOL_BF16
+
+
 def test_decoding_batches_that_shrink_from_40_rows_to_one(tmp_path_factory):
     """40 sequences that end one after the other: decoding steps of 40 down to 1 row take the pipelined
     64-row tiles (above 32 rows), then the matrix-vector kernels with two and one row tile (K shared

@@ -261,6 +261,83 @@ def test_a_library_function_called_by_name(kn):
         kn.call("lq_no_such_kernel")
 
 
+def pack_by_hand(w):
+    """The packed order written out with views: 8 rows' slabs of 64 k side by side."""
+    n, k = w.shape
+    return w.view(n // 8, 8, k // 64, 64).permute(0, 2, 1, 3).contiguous().view(n, k)
+
+
+@pytest.mark.parametrize("n,k", [(2048, 512), (4096, 4096), (6144, 2048), (4096, 1792), (2056, 1024), (8192, 4160)])
+def test_a_packed_weight_gives_every_product_the_bits_of_the_dense_one(kn, n, k):
+    """Wide bfloat16 weights may be held with 8 rows' slabs of 64 k side by side.  Every kernel that can meet
+    such a weight (the balanced kernel up to 32 rows, the pipelined tiles beyond, whole or in shares of K, with
+    and without the SwiGLU epilogue, the pair around a norm) reads it and sums in the order it sums a dense one."""
+    bf = torch.bfloat16
+    w = rnd((n, k), 31, bf, 0.05)
+    pw = kn.pack_weight(w)
+    assert getattr(pw, "packed", False) and tuple(pw.shape) == (n, k) and pw.dtype == bf
+    assert torch.equal(pw.data, pack_by_hand(w))
+    assert kn.pack_weight(pw) is pw
+    for m in (1, 8, 16, 17, 32, 33, 48, 64, 65, 128, 200, 256, 257, 512, 700, 1024, 2048):
+        x = rnd((m, k), 32 + m, bf)
+        pieces = kn.linear_pieces(bf, m, n, k)
+        shape = (pieces, m, n) if pieces > 1 else (m, n)
+        a = torch.full(shape, 7.0, dtype=torch.float32, device=DEV)
+        b = torch.full(shape, 9.0, dtype=torch.float32, device=DEV)
+        kn.linear(x, w, a)
+        kn.linear(x, pw, b)
+        assert torch.equal(a, b), (m, "float32 out", pieces)
+        a16 = torch.zeros((m, n), dtype=bf, device=DEV)
+        b16 = torch.ones((m, n), dtype=bf, device=DEV)
+        kn.linear(x, w, a16)
+        kn.linear(x, pw, b16)
+        assert torch.equal(a16, b16), (m, "bfloat16 out")
+        if n % 16 == 0:
+            a16 = torch.zeros((m, n // 2), dtype=bf, device=DEV)
+            b16 = torch.ones((m, n // 2), dtype=bf, device=DEV)
+            kn.linear_swiglu(x, w, a16)
+            kn.linear_swiglu(x, pw, b16)
+            assert torch.equal(a16, b16), (m, "swiglu")
+        parts = kn.linear_fused_parts(bf, m, n, k)
+        if parts > 0:
+            gain = 1 + 0.3 * rnd((n,), 33)
+            res = []
+            for weight in (w, pw):
+                stream = rnd((m, n), 34)
+                sq = torch.zeros((m, parts), dtype=torch.float32, device=DEV)
+                scaled = torch.zeros((m, n), dtype=bf, device=DEV)
+                kn.linear_residual(x, weight, stream, sq, gain=gain, scaled=scaled)
+                res.append((stream, sq, scaled))
+            assert all(torch.equal(p, q) for p, q in zip(*res)), (m, "residual")
+            sq_in = rnd((m, 5), 35).abs() * k
+            for swiglu in ((False, True) if n % 16 == 0 else (False,)):
+                outs = [torch.zeros((m, n // 2 if swiglu else n), dtype=bf, device=DEV) for _ in range(2)]
+                kn.linear_scaled(x, sq_in, 1e-5, w, outs[0], swiglu=swiglu)
+                kn.linear_scaled(x, sq_in, 1e-5, pw, outs[1], swiglu=swiglu)
+                assert torch.equal(outs[0], outs[1]), (m, "scaled", swiglu)
+    # a table that is also a head: the embedding reads the packed rows
+    toks = i32([5, n - 1, 0, 8, 7, -1, n])
+    a = torch.empty((7, k), dtype=torch.float32, device=DEV)
+    b = torch.empty((7, k), dtype=torch.float32, device=DEV)
+    kn.embed(w, toks, a)
+    kn.embed(pw, toks, b)
+    assert torch.equal(a, b)
+
+
+def test_weights_that_no_packed_reader_would_take_stay_dense(kn):
+    bf = torch.bfloat16
+    for shape, dtype in (((2048, 520), bf), ((2052, 512), bf), ((1024, 4096), bf), ((4096, 448), bf),
+                         ((4096, 4096), torch.float32)):
+        w = rnd(shape, 36, dtype)
+        assert kn.pack_weight(w) is w
+    kn.pack_weights = False
+    try:
+        w = rnd((4096, 4096), 37, bf)
+        assert kn.pack_weight(w) is w
+    finally:
+        kn.pack_weights = True
+
+
 def test_linear_bfloat16_odd_k_takes_the_generic_kernel(kn):
     x, w = rnd((9, 77), 14, torch.bfloat16), rnd((33, 77), 15, torch.bfloat16)
     out = torch.empty((9, 33), dtype=torch.float32, device=DEV)
