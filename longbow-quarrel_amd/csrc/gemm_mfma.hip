@@ -12,7 +12,7 @@
 //  * tiled, pipelined: 4 or 8 waves compute a 128 x 256 or 256 x 256 tile; operand slabs go from
 //    memory straight into a ring of LDS stages (no registers in between).  For many rows (prefill)
 //    and K a multiple of 32.  The same kernel with tiles of 64, 128 or 256 rows by 128, 64 or 32
-//    columns and three or four stages takes 33 to 256 rows of a wide matrix (long decoding batches,
+//    columns and three or four stages takes 13 to 256 rows of a wide matrix (long decoding batches,
 //    short prompts): the tile covers all rows, so every weight is read once, at streaming speed.
 //  * tiled: a block of 4 waves (2 x 2) computes a (2*WM*32) x (2*WN*32) tile, operands staged
 //    through padded LDS in steps of 64 k, next step prefetched into registers while the current one
@@ -998,14 +998,20 @@ int tiled_splits(int M, int N, int K) {
   return splits;
 }
 
-// ---- 33 to 256 rows of a wide matrix: the weights are what is read, once, at the speed of the memory.
+// ---- 13 to 256 rows of a wide matrix: the weights are what is read, once, at the speed of the memory.
 // The pipelined kernel streams them best (transfers of three or four slabs in flight, no registers in
 // between) when its tile covers all rows, so that a weight is read once, and is narrow enough, with K shared
 // out over blocks, for about one block a compute unit: 64 x 128 (8 waves), 128 x 128 (8 waves) or 256 x 128
 // tiles (8 waves) of 4, 4 and 3 stages.  A product that must come out whole (16-bit out: its consumer adds no
 // pieces) and has few columns takes the 64- or 32-column sibling instead.
+// (from 13 rows: with packed weights the tiles stream as fast as the matrix-vector kernels, whose time grows
+// with every row beyond 8; 8B shape, a decoding step at batch 12 4.10 ms either way, at batch 16 4.30 -> 4.13, at
+// batch 24 4.55 -> 4.10, at batch 32 4.74 -> 4.25)
+#ifndef LQ_MID_ROWS_FROM
+#define LQ_MID_ROWS_FROM 12
+#endif
 inline bool mid_rows(int M, int N, int K) {
-  return M > 32 && M <= 256 && K % 64 == 0 && K >= 512 && N >= 8 * lq_compute_units();
+  return M > LQ_MID_ROWS_FROM && M <= 256 && K % 64 == 0 && K >= 512 && N >= 8 * lq_compute_units();
 }
 
 inline int mid_splits_for(int tiles, int K) {
@@ -1150,7 +1156,7 @@ int lq_gemm_mfma_splits(int M, int N, int K) { return mfma_splits(M, N, K); }
 // rstd from those parts, optionally through the SwiGLU epilogue.  Both are the balanced kernel with one
 // row tile; lq_gemm_fused_parts says how many parts it leaves (0: this size is not taken).
 int lq_gemm_fused_parts(int M, int N, int K) {
-  if (M < 1 || M > 16 || !(N >= 8 * lq_compute_units() && K >= 512) || K % 8 != 0) return 0;
+  if (M < 1 || M > 16 || mid_rows(M, N, K) || !(N >= 8 * lq_compute_units() && K >= 512) || K % 8 != 0) return 0;
   int cols, grid;
   v3_runs(N, lq_compute_units(), 8, cols, grid);
   return grid;
