@@ -979,7 +979,7 @@ int pick_skinny(const void* x, const void* w, void* out, int M, int N, int K, in
   return launch_skinny<16, MT, EPI, TO>(x, w, out, M, N, K, lda, ldw, ldc, stream);
 }
 
-// A weight may be kept packed (8 rows' slabs of 64 k side by side, see lq_gemm_pack_layout) if every product
+// A weight may be kept packed (8 rows' slabs of 64 k side by side, see lq_pack_weight) if every product
 // with it runs in the pipelined kernel with slabs of 64 k or in the balanced kernel: wide, K in 64s.
 inline bool gemm_packable(int N, int K) {
   return N >= 8 * lq_compute_units() && N % 8 == 0 && K >= 512 && K % 64 == 0;
