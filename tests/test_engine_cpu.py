@@ -102,6 +102,49 @@ def test_a_step_knows_when_every_row_is_wanted_in_order(tmp_path):
     assert seen == [True, False, False, True]
 
 
+def test_every_product_weight_is_offered_to_the_kernels_once_when_weights_are_bound(tmp_path):
+    """A kernel object with `pack_weight` is asked once for each matrix of a product (q, k and v as one, o, gate and
+    up as one, down, the head), and what it hands back is what the parts keep; a tied table is offered once and then
+    serves the embedding and the head.  One without the method gets dense tensors, as the stand-in of these tests."""
+    class Marked(torch.Tensor):
+        pass
+
+    class Packing(CpuKernels):
+        def __init__(self):
+            super().__init__()
+            self.offered = []
+
+        def pack_weight(self, w):
+            self.offered.append(tuple(w.shape))
+            return w.as_subclass(Marked)
+
+    for cfg in (TINY_A, TINY_B):
+        folder = write_folder(tmp_path / ("tied" if cfg["tie_word_embeddings"] else "untied"), cfg, seed=2)
+        kn = Packing()
+        eng = lq.load_engine(folder, dtype="float32", max_tokens=256, device="cpu", kernels=kn)
+        m = eng.model
+        layers, width, inner = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
+        hd = cfg.get("head_dim") or width // cfg["num_attention_heads"]
+        qkv = (cfg["num_attention_heads"] + 2 * cfg["num_key_value_heads"]) * hd
+        want = [(qkv, width), (width, cfg["num_attention_heads"] * hd), (2 * inner, width), (width, inner)] * layers
+        want.append((cfg["vocab_size"], width))
+        assert sorted(kn.offered) == sorted(want)
+        for b in m.blocks:
+            assert all(isinstance(w, Marked) for w in (b.mixer.w_qkv, b.mixer.w_o, b.ffn.w_gate_up, b.ffn.w_down))
+        assert isinstance(m.head, Marked)
+        if cfg["tie_word_embeddings"]:
+            assert m.head is m.embedding.table
+        else:
+            assert not isinstance(m.embedding.table, Marked)
+        # and the engine still gives the plain implementation's logits
+        c, tensors = read_folder(folder)
+        toks = random_tokens(9, cfg["vocab_size"], 4)
+        s = eng.new_sequence()
+        got = eng.step([StepEntry(s, toks, range(9))])
+        eng.release(s)
+        assert rel_err(got, plain.PlainLlama(c, tensors).forward(toks, plain.identity)) < 1e-5
+
+
 def test_a_released_slot_leaves_no_trace(tmp_path):
     eng, ref = make(tmp_path, TINY_C, max_tokens=256)
     first = random_tokens(130, 331, 3)
