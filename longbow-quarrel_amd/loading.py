@@ -48,7 +48,8 @@ def load_engine(folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_to
     model = DecoderModel(spec_from_config(config))
     env = _env(dtype, device, kernels)
     tensors = load_tensors(folder, model.tensor_specs(), env.dtype, env.device)
-    model.bind(tensors, env)
+    model.bind(tensors, env, consume=True)
+    del tensors
     engine = Engine(model, env, max_tokens, max_slots, max_sequence_tokens)
     engine.config = config
     return engine
@@ -67,7 +68,8 @@ def random_engine(config: ModelConfig, seed: int, dtype: Union[str, torch.dtype]
         if s.kind == "vector32":
             tensors[s.name] = tensors[s.name].float()
     check_names_and_shapes(specs, {n: tuple(t.shape) for n, t in tensors.items()}, "random weights")
-    model.bind(tensors, env)
+    model.bind(tensors, env, consume=True)
+    del tensors
     engine = Engine(model, env, max_tokens, max_slots, max_sequence_tokens)
     engine.config = config
     return engine

@@ -89,13 +89,25 @@ class DecoderModel:
             specs.extend(self.logits_step.tensor_specs())
         return specs
 
-    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv, consume: bool = False) -> None:
+        """Hands every part its tensors.  With `consume` (tensors a dict that the caller gives up) a part's
+        tensors leave the dict as soon as the part is bound: what a part keeps in another form (a packed
+        product weight, q, k and v as one matrix) then frees its source at once, and binding a model takes the
+        room of its weights plus a layer's, not twice its weights."""
         self.env = env
         s = self.spec
+        waiting: Dict[str, int] = {}  # parts that still have to see a tensor (two parts may name one)
+        for p in self.parts():
+            for spec in p.tensor_specs():
+                waiting[spec.name] = waiting.get(spec.name, 0) + 1
         for p in self.parts():
             p.bind(tensors, env)
+            for spec in p.tensor_specs():
+                waiting[spec.name] -= 1
+                if consume and waiting[spec.name] == 0:
+                    tensors.pop(spec.name, None)
         if s.head_name is not None and not s.tie_head:
-            self.head = product_weight(env, tensors[s.head_name])
+            self.head = product_weight(env, tensors.pop(s.head_name) if consume else tensors[s.head_name])
         else:
             # the head is the embedding when the file has none: internal/engine/engine.go:1106-1116
             table = self.embedding.table

@@ -131,6 +131,15 @@ def test_every_product_weight_is_offered_to_the_kernels_once_when_weights_are_bo
         assert sorted(kn.offered) == sorted(want)
         for b in m.blocks:
             assert all(isinstance(w, Marked) for w in (b.mixer.w_qkv, b.mixer.w_o, b.ffn.w_gate_up, b.ffn.w_down))
+        # a dict that the caller gives up is emptied part by part; one that it keeps is left alone
+        from longbow_quarrel_amd.model import DecoderModel
+        from longbow_quarrel_amd.registry import spec_from_config
+        for consume in (True, False):
+            again = DecoderModel(spec_from_config(eng.config))
+            given = dict(read_folder(folder)[1])
+            count = len(given)
+            again.bind(given, eng.env, consume=consume)
+            assert len(given) == (0 if consume else count)
         assert isinstance(m.head, Marked)
         if cfg["tie_word_embeddings"]:
             assert m.head is m.embedding.table

@@ -422,6 +422,25 @@ def test_packed_weights_and_a_packed_tied_table_give_the_bits_of_dense_ones(tmp_
             assert rel_err(outs[0][:n], ref.forward(prompt[:n], plain.round_bf16)) < TOL_BF16
 
 
+def test_loading_a_model_takes_the_room_of_its_weights_and_a_layer_more(tmp_path_factory):
+    """Weights that a part keeps in another form (packed, q k and v as one matrix, gate and up interleaved) give
+    their source back as soon as the part is bound: the most memory in use while a model loads stays near what
+    the loaded model holds, not twice that (a 70B shape's 141 GB would not fit twice)."""
+    cfg = dict(WIDE, intermediate_size=2304, num_hidden_layers=8, vocab_size=2056)
+    folder = write_folder(tmp_path_factory.mktemp("room"), cfg, seed=7, std=0.03)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    before = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    eng = lq.load_engine(folder, dtype="bfloat16", max_tokens=64)
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated() - before
+    most = torch.cuda.max_memory_allocated() - before
+    layer = held / cfg["num_hidden_layers"]
+    assert getattr(eng.model.blocks[0].mixer.w_qkv, "packed", False)
+    assert most < held + 2.5 * layer, (held, most)
+
+
 def test_decoding_batches_that_shrink_from_40_rows_to_one(tmp_path_factory):
     """40 sequences that end one after the other: decoding steps of 40 down to 1 row take the pipelined
     64-row tiles (above 12 rows: K shared between blocks, the pieces added by the norms), then the
