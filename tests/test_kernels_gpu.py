@@ -272,7 +272,8 @@ def pack_by_hand(w):
     return w.view(n // 8, 8, k // 64, 64).permute(0, 2, 1, 3).contiguous().view(n, k)
 
 
-@pytest.mark.parametrize("n,k", [(2048, 512), (4096, 4096), (6144, 2048), (4096, 1792), (2056, 1024), (8192, 4160)])
+@pytest.mark.parametrize("n,k", [(2048, 512), (4096, 4096), (6144, 2048), (4096, 1792), (2056, 1024), (8192, 4160),
+                                 (28672, 4096)])
 def test_a_packed_weight_gives_every_product_the_bits_of_the_dense_one(kn, n, k):
     """Wide bfloat16 weights may be held with 8 rows' slabs of 64 k side by side.  Every kernel that can meet
     such a weight (the balanced kernel up to 32 rows, the pipelined tiles beyond, whole or in shares of K, with
